@@ -1,0 +1,120 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+A batch holds, for each of its requests, a run of that request's next tokens:
+a whole prompt, a portion of one cut anywhere, or one decoded token; all runs
+of a step form one flat batch.  The step runs only the tokens it is given,
+against the pages that earlier steps wrote, writes these tokens' keys and values,
+and returns float32 logits at the places asked for.
+
+The reference has two runners instead, which it calls back to back and never
+mixes: whole right-padded prompts (``serving/prefill.py:60-76``) and single
+decoded tokens (``serving/paged_decoder.py:364-408``).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..parts.context import StepContext
+from ..parts.model import DecoderModel
+
+
+@dataclass
+class StepEntry:
+    req: int                         # the request's id in the cache manager
+    tokens: Sequence[int]            # its next tokens, in order
+    want: Sequence[int] = field(default_factory=list)  # places among ``tokens`` whose logits are wanted
+
+
+class StepRunner:
+    def __init__(self, model: DecoderModel, cache: CacheManager, kernels, device, max_positions: int):
+        self.model = model
+        self.cache = cache
+        self.kernels = kernels
+        self.device = torch.device(device)
+        self.max_positions = max_positions
+        self.vocab_size = model.vocab_size
+
+    def _check(self, entries: List[StepEntry]) -> None:
+        seen = set()
+        for e in entries:
+            if e.req in seen:
+                raise ValueError(f"request {e.req} appears twice in one step")
+            seen.add(e.req)
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.req} brings no tokens")
+            if e.req not in self.cache.lengths:
+                raise KeyError(f"request {e.req} is not admitted to the cache")
+            if self.cache.lengths[e.req] + len(e.tokens) > self.max_positions:
+                raise ValueError(
+                    f"request {e.req} would reach position {self.cache.lengths[e.req] + len(e.tokens)}, "
+                    f"beyond the engine's {self.max_positions}")
+            for t in e.tokens:
+                if not 0 <= int(t) < self.vocab_size:
+                    raise ValueError(f"token id {t} of request {e.req} is outside [0, {self.vocab_size})")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise ValueError(f"wanted place {w} of request {e.req} is outside its {len(e.tokens)} tokens")
+
+    def build_context(self, entries: List[StepEntry]) -> StepContext:
+        """Takes the pages the step needs and lays its metadata out on the device."""
+        self._check(entries)
+        cache = self.cache
+        n_seqs = len(entries)
+        q_lens = [len(e.tokens) for e in entries]
+        n_tokens = sum(q_lens)
+        starts = [cache.extend(e.req, len(e.tokens)) for e in entries]
+        n_groups = len(cache.groups)
+        reqs = [e.req for e in entries]
+        width = max(1, cache.max_table_len(reqs))
+        n_rows = sum(len(e.want) for e in entries)
+
+        sizes = [n_tokens, n_tokens, n_tokens, n_seqs + 1, n_seqs, n_seqs, max(n_rows, 1)] + \
+                [n_seqs * width] * n_groups
+        offsets = np.concatenate([[0], np.cumsum(sizes)])
+        host = np.empty(int(offsets[-1]), dtype=np.int32)
+        tok, pos, sot, cu, kvl, slots, rows = (host[offsets[i]:offsets[i + 1]] for i in range(7))
+        cu[0] = 0
+        rows[:] = 0
+        t = r = 0
+        for s, e in enumerate(entries):
+            n = q_lens[s]
+            tok[t:t + n] = e.tokens
+            pos[t:t + n] = np.arange(starts[s], starts[s] + n, dtype=np.int32)
+            sot[t:t + n] = s
+            for w in e.want:
+                rows[r] = t + int(w)
+                r += 1
+            t += n
+            cu[s + 1] = t
+            kvl[s] = starts[s] + n
+            slots[s] = cache.slot(e.req)
+        for g in range(n_groups):
+            tab = host[offsets[7 + g]:offsets[8 + g]].reshape(n_seqs, width)
+            tab[:] = -1
+            for s, e in enumerate(entries):
+                row = cache.table(g, e.req)
+                tab[s, :len(row)] = row
+
+        dev = torch.from_numpy(host).to(self.device)
+        part = lambda i: dev[int(offsets[i]):int(offsets[i + 1])]
+        ctx = StepContext(
+            n_tokens=n_tokens, n_seqs=n_seqs,
+            token_ids=part(0), positions=part(1), seq_of_token=part(2), cu_q=part(3), kv_len=part(4),
+            state_slots=part(5), logit_rows=part(6)[:n_rows] if n_rows else None, n_logit_rows=n_rows,
+            max_q_len=max(q_lens), max_kv_len=int(kvl.max()), kernels=self.kernels,
+        )
+        ctx.block_tables = [part(7 + g).view(n_seqs, width) for g in range(n_groups)]
+        return ctx
+
+    @torch.no_grad()
+    def run(self, entries: List[StepEntry]) -> Optional[torch.Tensor]:
+        """Runs one step; returns float32 logits ``[wanted, vocab]`` in the order of entries and wants."""
+        ctx = self.build_context(entries)
+        caches = self.cache.layer_caches(ctx.block_tables)
+        return self.model.forward(ctx, caches)

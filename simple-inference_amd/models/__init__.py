@@ -1,0 +1,1 @@
+from . import llama  # noqa: F401  (registers LlamaForCausalLM)

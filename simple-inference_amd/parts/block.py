@@ -1,0 +1,26 @@
+"""The arrangement of parts in a layer.
+
+Pre-norm (reference: ``model/block.py:135-147``):
+``x += mixer(norm1(x))``; ``x += feed_forward(norm2(x))``.  Each add is carried
+as the stream's pending delta and summed into the float32 residual by the norm
+that follows (the next layer's, or the model's last norm).
+"""
+
+from __future__ import annotations
+
+from .registry import register_block
+
+
+@register_block("prenorm")
+class PreNormBlock:
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.feed_forward_norm = feed_forward_norm
+
+    def forward(self, stream, ctx, cache):
+        h = self.mixer_norm.forward(stream)
+        stream.delta = self.mixer.forward(h, ctx, cache)
+        h = self.feed_forward_norm.forward(stream)
+        stream.delta = self.feed_forward.forward(h, ctx)

@@ -1,0 +1,38 @@
+"""Root-mean-square norm (reference: ``ops/rmsnorm.py:41-46``, ``kernels/rmsnorm_kernel.py:105-113``).
+
+``y = x * rsqrt(mean(x^2) + eps) * w`` with the statistic, the normalisation and
+the gain in float32 and one rounding to the compute dtype, as the reference's
+fused kernel does.  The add of the pending residual delta is fused in front.
+"""
+
+from __future__ import annotations
+
+from .plan import TensorSpec
+from .registry import register_norm
+
+
+@register_norm("rmsnorm")
+class RMSNorm:
+    def __init__(self, params, env):
+        self.size = int(params["size"])
+        self.eps = float(params["eps"])
+        self.env = env
+        self.weight = None
+
+    def weight_specs(self):
+        return {"weight": TensorSpec((self.size,), "vector")}
+
+    def bind(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, stream, rows=None):
+        """Adds ``stream.delta`` into ``stream.residual`` and returns the normed rows.
+
+        With ``rows`` (int32 indices) only those rows are computed and the residual
+        is left as it was: that form ends a forward pass.
+        """
+        out = self.env.kernels.add_rmsnorm(
+            stream.residual, stream.delta, self.weight, self.eps, self.env.dtype, rows)
+        if rows is None:
+            stream.delta = None
+        return out

@@ -1,0 +1,90 @@
+"""The data that describes a model: which parts each layer has and how layers run.
+
+A ``ModelPlan`` is plain data.  An architecture's ``build_plan`` writes it from
+its configuration; ``DecoderModel`` builds the parts it names.  Nothing in a plan
+refers to a concrete architecture: a part is named by its ``kind`` (a key of the
+part registries), its sizes and constants are in ``params``, and ``weights`` maps
+the part's own tensor names to the names in the checkpoint.
+
+* Layers may differ from one another: every ``LayerSpec`` names its own mixer,
+  feed-forward and norms.
+* ``order`` lists layer indices in the order they run.  A layer may be named
+  twice (each run keeps a cache of its own), and a mixer may read the cache
+  that another layer's latest run wrote (``params["kv_from_layer"]``).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional, Tuple
+
+
+@dataclass
+class PartSpec:
+    kind: str
+    params: Dict[str, Any] = field(default_factory=dict)
+    weights: Dict[str, str] = field(default_factory=dict)
+
+
+@dataclass
+class LayerSpec:
+    mixer: PartSpec
+    feed_forward: PartSpec
+    mixer_norm: PartSpec
+    feed_forward_norm: PartSpec
+    block: str = "prenorm"
+
+
+@dataclass
+class ModelPlan:
+    hidden_size: int
+    vocab_size: int
+    embedding: PartSpec
+    layers: List[LayerSpec]
+    final_norm: PartSpec
+    head: PartSpec
+    order: Optional[List[int]] = None  # None → every layer once, in index order
+    bos_token_id: Optional[int] = None
+    eos_token_ids: Tuple[int, ...] = ()
+    max_position_embeddings: Optional[int] = None
+
+    def run_order(self) -> List[int]:
+        order = list(range(len(self.layers))) if self.order is None else list(self.order)
+        for i in order:
+            if not 0 <= i < len(self.layers):
+                raise ValueError(f"order names layer {i}, but the plan has {len(self.layers)} layers")
+        return order
+
+
+# ---------------------------------------------------------------------------
+# What a part asks of the loader and of the cache manager
+# ---------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """Shape and role of one tensor a part reads from the checkpoint.
+
+    role "matrix": kept in the engine's compute dtype (bfloat16 or float32).
+    role "vector": small gains and the like, held in float32 in both modes.
+    role "table":  integers, held as int32.
+    """
+
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+
+
+@dataclass(frozen=True)
+class PagedKVNeed:
+    """Keys and values in pages: all keys (``window`` None) or the last ``window``."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size (one row per running request)."""
+
+    shape: Tuple[int, ...]
+    dtype: str = "float32"

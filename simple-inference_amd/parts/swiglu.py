@@ -1,0 +1,43 @@
+"""Dense gated feed-forward (reference: ``ops/mlp.py:87-128``).
+
+``y = (silu(h Wg^T) * (h Wu^T)) Wd^T``.  Gate and up are stacked into one
+``[2I, H]`` matrix at load (reference: ``ops/mlp.py:104``) so one product gives
+both; ``silu(g) * u`` is computed in float32 and rounded once (reference:
+``kernels/swiglu_kernel.py:142-150``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .plan import TensorSpec
+from .registry import register_feed_forward
+
+
+@register_feed_forward("swiglu")
+class SwiGLU:
+    """params: hidden_size, intermediate_size."""
+
+    def __init__(self, params, env):
+        self.hidden = int(params["hidden_size"])
+        self.inter = int(params["intermediate_size"])
+        self.env = env
+        self.w_gate_up = None
+        self.w_down = None
+
+    def weight_specs(self):
+        return {
+            "gate": TensorSpec((self.inter, self.hidden)),
+            "up": TensorSpec((self.inter, self.hidden)),
+            "down": TensorSpec((self.hidden, self.inter)),
+        }
+
+    def bind(self, tensors):
+        self.w_gate_up = torch.cat([tensors["gate"], tensors["up"]], dim=0).contiguous()
+        self.w_down = tensors["down"].contiguous()
+
+    def forward(self, h, ctx):
+        k = self.env.kernels
+        gu = k.linear(h, self.w_gate_up)
+        a = k.swiglu(gu)
+        return k.linear(a, self.w_down)
