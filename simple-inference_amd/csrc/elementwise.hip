@@ -1,0 +1,137 @@
+// Embedding gather, residual add + RMS norm, SwiGLU activation.
+//
+// These are bound by memory traffic or by launch latency.  The residual stream is float
+// in both modes; rows are handled by one workgroup each, with vector accesses where the
+// row length allows.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------
+// Embedding: out[n, :] = float(table[ids[n], :])          (reference: ops/embedding.py:57-60)
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                             float* __restrict__ out, int hidden) {
+    const int n = blockIdx.x;
+    const T* src = table + (size_t)ids[n] * hidden;
+    float* dst = out + (size_t)n * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+}
+
+SIA_EXPORT int sia_embed(const int* ids, const void* table, float* out, int n_tokens, int hidden,
+                         int table_dtype, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    dim3 grid(n_tokens), block(256);
+    if (table_dtype == SIA_F32)
+        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, (const float*)table, out, hidden);
+    else if (table_dtype == SIA_BF16)
+        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, (const bf16_t*)table, out, hidden);
+    else
+        return SIA_BAD_ARGUMENT;
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// Residual add + RMS norm  (reference: ops/rmsnorm.py:41-46, kernels/rmsnorm_kernel.py:105-113)
+//
+//   x = residual[row] + delta[row]            (float; delta may be absent)
+//   y = x * rsqrt(mean(x^2) + eps) * w        (float, one rounding to the output type)
+//
+// rows == nullptr: every row r of the batch; x is written back into residual[r].
+// rows != nullptr: out[i] comes from row rows[i]; residual is not written.
+// The sum of squares is reduced in a fixed order that depends on the row length only.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                   const float* __restrict__ weight, T* __restrict__ out,
+                                   const int* __restrict__ rows, int hidden, float eps) {
+    __shared__ float scratch[16];
+    const int i_out = blockIdx.x;
+    const int row = rows ? rows[i_out] : i_out;
+    float* res = residual + (size_t)row * hidden;
+    const T* del = delta ? delta + (size_t)row * hidden : nullptr;
+    T* dst = out + (size_t)i_out * hidden;
+
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float x = res[i];
+        if (del) x += to_float(del[i]);
+        if (!rows && del) res[i] = x;
+        ss += x * x;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = rsqrtf(ss / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float x = res[i];
+        if (rows && del) x += to_float(del[i]);
+        dst[i] = from_float<T>(x * inv * weight[i]);
+    }
+}
+
+SIA_EXPORT int sia_add_rmsnorm(float* residual, const void* delta, const float* weight, void* out,
+                               const int* rows, int n_out, int hidden, float eps, int dtype,
+                               hipStream_t stream) {
+    if (n_out <= 0) return 0;
+    dim3 grid(n_out), block(hidden >= 2048 ? 512 : 256);
+    if (dtype == SIA_F32)
+        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, stream, residual, (const float*)delta,
+                           weight, (float*)out, rows, hidden, eps);
+    else if (dtype == SIA_BF16)
+        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, grid, block, 0, stream, residual, (const bf16_t*)delta,
+                           weight, (bf16_t*)out, rows, hidden, eps);
+    else
+        return SIA_BAD_ARGUMENT;
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// SwiGLU: out[n, i] = silu(gu[n, i]) * gu[n, I + i], silu(g) = g / (1 + exp(-g)), in float
+// (reference: ops/mlp.py:117-128, kernels/swiglu_kernel.py:142-150)
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
+    const int n = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= inter) return;
+    const T* row = gu + (size_t)n * 2 * inter;
+    const float g = to_float(row[i]);
+    const float u = to_float(row[inter + i]);
+    out[(size_t)n * inter + i] = from_float<T>(g / (1.f + expf(-g)) * u);
+}
+
+SIA_EXPORT int sia_swiglu(const void* gu, void* out, int n_tokens, int inter, int dtype, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (n_tokens > 65535) return SIA_BAD_ARGUMENT;
+    dim3 block(256), grid((inter + 255) / 256, n_tokens);
+    if (dtype == SIA_F32)
+        hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)out, inter);
+    else if (dtype == SIA_BF16)
+        hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)out, inter);
+    else
+        return SIA_BAD_ARGUMENT;
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// Casts between the two element types (used where a float32-stored matrix meets bfloat16
+// activations).
+// ---------------------------------------------------------------------------------------
+__global__ void cast_bf16_to_f32_kernel(const bf16_t* __restrict__ in, float* __restrict__ out, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = bf16_to_float(in[i]);
+}
+__global__ void cast_f32_to_bf16_kernel(const float* __restrict__ in, bf16_t* __restrict__ out, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = float_to_bf16(in[i]);
+}
+
+SIA_EXPORT int sia_cast(const void* in, void* out, long long n, int in_dtype, hipStream_t stream) {
+    if (n <= 0) return 0;
+    dim3 block(256), grid((unsigned)((n + 255) / 256));
+    if (in_dtype == SIA_BF16)
+        hipLaunchKernelGGL(cast_bf16_to_f32_kernel, grid, block, 0, stream, (const bf16_t*)in, (float*)out, (size_t)n);
+    else if (in_dtype == SIA_F32)
+        hipLaunchKernelGGL(cast_f32_to_bf16_kernel, grid, block, 0, stream, (const float*)in, (bf16_t*)out, (size_t)n);
+    else
+        return SIA_BAD_ARGUMENT;
+    return SIA_LAUNCH_CHECK();
+}

@@ -1,0 +1,249 @@
+"""The device kernels, as an object the parts call.
+
+``HipKernels`` loads the compiled HIP libraries and launches their entry points on
+torch's current stream, with torch tensors as buffers.  It checks on the host that
+operand shapes, dtypes and devices are what the kernels and their grids assume, and
+raises before a launch that would not fit.  There is no other implementation in this
+package: without a GPU or without ``hipcc`` to build a missing library it raises.
+Matrix products of the bfloat16 path go to the BLAS library through ``torch``, as the
+reference's go to its vendor's (``ops/attention.py:128-130``, ``ops/mlp.py:117,128``);
+the 32-bit path uses this package's own float kernel.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+_c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
+
+_SIGNATURES = {
+    "sia_embed": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "sia_swiglu": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_cast": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
+    "sia_rope_kv_write": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
+                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_attention_generic": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "sia_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_sample": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _bind(lib, signatures):
+    for name, argtypes in signatures.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_int
+
+
+class HipKernels:
+    name = "hip-gfx950"
+
+    def __init__(self, device="cuda:0"):
+        if not torch.cuda.is_available():
+            raise KernelError(
+                "simple-inference_amd needs an AMD GPU: torch sees no device, and the engine has no "
+                "other implementation of its kernels")
+        self.device = torch.device(device)
+        self.core = build.load_library("core")
+        _bind(self.core, _SIGNATURES)
+
+    # -- helpers -------------------------------------------------------------
+    def _stream(self):
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def _check(self, code: int, what: str):
+        if code != 0:
+            if code == 10001:
+                raise KernelError(f"{what}: the kernel refused its arguments (sizes or types it does not take)")
+            raise KernelError(f"{what}: HIP error {code}")
+
+    def _want(self, t: torch.Tensor, what: str, dtype=None, shape=None):
+        if t.device.type != "cuda":
+            raise KernelError(f"{what} must be on the GPU, is on {t.device}")
+        if not t.is_contiguous():
+            raise KernelError(f"{what} must be contiguous")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{what} must be {dtype}, is {t.dtype}")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{what} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+
+    # -- embedding -------------------------------------------------------------
+    def embed(self, token_ids, table):
+        self._want(token_ids, "token_ids", torch.int32)
+        self._want(table, "embedding table")
+        if table.dtype not in _DT or table.dim() != 2:
+            raise KernelError(f"embedding table must be a float32 or bfloat16 matrix, is {table.dtype} {tuple(table.shape)}")
+        n, hidden = token_ids.numel(), table.shape[1]
+        out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
+        self._check(self.core.sia_embed(_ptr(token_ids), _ptr(table), _ptr(out), n, hidden, _DT[table.dtype],
+                                        self._stream()), "embed")
+        return out
+
+    # -- residual add + rms norm ---------------------------------------------
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None):
+        n, hidden = residual.shape
+        self._want(residual, "residual", torch.float32)
+        self._want(weight, "norm weight", torch.float32, (hidden,))
+        if out_dtype not in _DT:
+            raise KernelError(f"norm output dtype {out_dtype} is not float32 or bfloat16")
+        if delta is not None:
+            self._want(delta, "delta", out_dtype, (n, hidden))
+        n_out = n
+        if rows is not None:
+            self._want(rows, "rows", torch.int32)
+            n_out = rows.numel()
+        out = torch.empty((n_out, hidden), dtype=out_dtype, device=residual.device)
+        self._check(self.core.sia_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows),
+                                              n_out, hidden, float(eps), _DT[out_dtype], self._stream()),
+                    "add_rmsnorm")
+        return out
+
+    # -- matrix product --------------------------------------------------------
+    def linear(self, x, w, out_float32=False):
+        """``x [M, K] @ w [N, K]^T`` with float accumulation."""
+        self._want(x, "linear input")
+        self._want(w, "linear weight")
+        if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+            raise KernelError(f"linear shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}")
+        if x.dtype not in _DT or w.dtype not in _DT:
+            raise KernelError(f"linear takes float32 or bfloat16, got {x.dtype} and {w.dtype}")
+        M, K = x.shape
+        N = w.shape[0]
+        if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+            y = torch.mm(x, w.t())  # BLAS library, float accumulation
+            return y.float() if out_float32 else y
+        # True 32-bit product.  A float32-stored matrix meeting bfloat16 activations widens them.
+        back = None
+        if x.dtype == torch.bfloat16:
+            back = torch.bfloat16
+            x = self.cast(x, torch.float32)
+        if w.dtype == torch.bfloat16:
+            w = self.cast(w, torch.float32)
+        y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+        self._check(self.core.sia_gemm_generic(_ptr(x), _ptr(w), _ptr(y), M, N, K, 0, 1, self._stream()),
+                    "gemm_generic")
+        if back is not None and not out_float32:
+            y = self.cast(y, back)
+        return y
+
+    def gemm_generic(self, x, w, out_float32=False):
+        """The plain kernel for either dtype (tests compare it with the library product)."""
+        self._want(x, "gemm input")
+        self._want(w, "gemm weight", x.dtype)
+        M, K = x.shape
+        N = w.shape[0]
+        out_dtype = torch.float32 if (out_float32 or x.dtype == torch.float32) else x.dtype
+        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        self._check(self.core.sia_gemm_generic(_ptr(x), _ptr(w), _ptr(y), M, N, K, _DT[x.dtype],
+                                               int(out_dtype == torch.float32), self._stream()), "gemm_generic")
+        return y
+
+    def cast(self, x, dtype):
+        self._want(x, "cast input")
+        if x.dtype == dtype:
+            return x
+        if {x.dtype, dtype} != {torch.float32, torch.bfloat16}:
+            raise KernelError(f"cast is between float32 and bfloat16 only, got {x.dtype} -> {dtype}")
+        out = torch.empty(x.shape, dtype=dtype, device=x.device)
+        self._check(self.core.sia_cast(_ptr(x), _ptr(out), x.numel(), _DT[x.dtype], self._stream()), "cast")
+        return out
+
+    # -- feed-forward activation ---------------------------------------------
+    def swiglu(self, gu):
+        self._want(gu, "swiglu input")
+        if gu.dtype not in _DT or gu.dim() != 2 or gu.shape[1] % 2:
+            raise KernelError(f"swiglu takes a [tokens, 2*intermediate] float32/bfloat16 matrix, got {gu.dtype} {tuple(gu.shape)}")
+        n, two_i = gu.shape
+        out = torch.empty((n, two_i // 2), dtype=gu.dtype, device=gu.device)
+        for n0 in range(0, n, 65535):  # grid.y limit
+            n1 = min(n, n0 + 65535)
+            self._check(self.core.sia_swiglu(_ptr(gu[n0:n1]), _ptr(out[n0:n1]), n1 - n0, two_i // 2,
+                                             _DT[gu.dtype], self._stream()), "swiglu")
+        return out
+
+    # -- rotation + cache write ------------------------------------------------
+    def rope_kv_write(self, qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache):
+        self._want(qkv, "qkv")
+        n, width = qkv.shape
+        if qkv.dtype not in _DT:
+            raise KernelError(f"qkv must be float32 or bfloat16, is {qkv.dtype}")
+        if width != (n_heads + 2 * n_kv_written) * head_dim:
+            raise KernelError(f"qkv row of {width} does not hold {n_heads} + 2*{n_kv_written} heads of {head_dim}")
+        if n != ctx.n_tokens:
+            raise KernelError(f"qkv has {n} rows, the step {ctx.n_tokens} tokens")
+        if rotary_dim:
+            for t, what in ((cos, "cos table"), (sin, "sin table")):
+                self._want(t, what, torch.float32)
+                if t.shape[1] != rotary_dim // 2 or t.shape[0] <= ctx.max_kv_len - 1:
+                    raise KernelError(f"{what} {tuple(t.shape)} does not cover position {ctx.max_kv_len - 1} "
+                                      f"with {rotary_dim // 2} pairs")
+        table = table_w = k_pages = v_pages = None
+        page_size = 0
+        if n_kv_written:
+            k_pages, v_pages, table, page_size = cache.k_pages, cache.v_pages, cache.block_table, cache.page_size
+            self._check_pages(k_pages, v_pages, table, page_size, n_kv_written, head_dim, qkv.dtype, ctx)
+        table_w = table.shape[1] if table is not None else 0
+        self._check(self.core.sia_rope_kv_write(
+            _ptr(qkv), width, _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None,
+            _ptr(ctx.positions), _ptr(ctx.seq_of_token), _ptr(table), table_w, _ptr(k_pages), _ptr(v_pages),
+            n, n_heads, n_kv_written, head_dim, rotary_dim, page_size, _DT[qkv.dtype], self._stream()),
+            "rope_kv_write")
+
+    def _check_pages(self, k_pages, v_pages, table, page_size, n_kv, head_dim, dtype, ctx):
+        self._want(k_pages, "key pages", dtype)
+        self._want(v_pages, "value pages", dtype)
+        pages = k_pages.shape[0]
+        if tuple(k_pages.shape) != (pages, n_kv, page_size, head_dim):
+            raise KernelError(f"key pages {tuple(k_pages.shape)} are not [pages, {n_kv}, {page_size}, {head_dim}]")
+        if tuple(v_pages.shape) != (pages, n_kv, head_dim, page_size):
+            raise KernelError(f"value pages {tuple(v_pages.shape)} are not [pages, {n_kv}, {head_dim}, {page_size}]")
+        self._want(table, "block table", torch.int32)
+        if table.dim() != 2 or table.shape[0] != ctx.n_seqs or table.shape[1] * page_size < ctx.max_kv_len:
+            raise KernelError(f"block table {tuple(table.shape)} does not cover {ctx.n_seqs} sequences of up to "
+                              f"{ctx.max_kv_len} positions with pages of {page_size}")
+
+    # -- attention ---------------------------------------------------------------
+    def paged_attention(self, qkv, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
+        self._want(qkv, "qkv")
+        n, width = qkv.shape
+        if width < n_heads * head_dim or n != ctx.n_tokens:
+            raise KernelError(f"qkv {tuple(qkv.shape)} does not hold {ctx.n_tokens} rows of {n_heads} heads of {head_dim}")
+        self._check_pages(cache.k_pages, cache.v_pages, cache.block_table, cache.page_size, n_kv_heads, head_dim,
+                          qkv.dtype, ctx)
+        out = torch.empty((n, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+        self._check(self.core.sia_attention_generic(
+            _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(cache.block_table),
+            cache.block_table.shape[1], _ptr(ctx.seq_of_token), _ptr(ctx.positions), _ptr(out), n, n_heads,
+            n_kv_heads, head_dim, cache.page_size, float(scale), int(window or 0), _DT[qkv.dtype],
+            self._stream()), "attention_generic")
+        return out
+
+    # -- sampling ------------------------------------------------------------------
+    def sample(self, logits, temperature, top_k, top_p, uniform):
+        rows, vocab = logits.shape
+        self._want(logits, "logits", torch.float32)
+        self._want(temperature, "temperature", torch.float32, (rows,))
+        self._want(top_k, "top_k", torch.int32, (rows,))
+        self._want(top_p, "top_p", torch.float32, (rows,))
+        self._want(uniform, "uniform", torch.float32, (rows,))
+        out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+        self._check(self.core.sia_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
+                                         _ptr(out), rows, vocab, self._stream()), "sample")
+        return out

@@ -1,0 +1,215 @@
+"""Each HIP kernel alone against its plain torch twin, at sizes other than the tiny models'."""
+
+import math
+
+import pytest
+import torch
+
+from twins import TwinKernels
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from simple_inference_amd.kernels import HipKernels
+    return HipKernels()
+
+
+twin = TwinKernels()
+
+
+def tol(dtype):
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-2)
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+class Ctx:
+    """The fields of a step context that the kernels read."""
+
+    def __init__(self, q_lens, kv_lens):
+        pos, sot, cu = [], [], [0]
+        for s, (q, kv) in enumerate(zip(q_lens, kv_lens)):
+            pos += list(range(kv - q, kv))
+            sot += [s] * q
+            cu.append(cu[-1] + q)
+        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+        self.positions, self.seq_of_token, self.cu_q, self.kv_len = i32(pos), i32(sot), i32(cu), i32(kv_lens)
+        self.n_tokens, self.n_seqs = len(pos), len(q_lens)
+        self.max_q_len, self.max_kv_len = max(q_lens), max(kv_lens)
+
+
+class Cache:
+    def __init__(self, n_pages, n_kv, page_size, head_dim, dtype, kv_lens, seed=0):
+        from types import SimpleNamespace
+        self.page_size = page_size
+        self.k_pages = torch.zeros(n_pages, n_kv, page_size, head_dim, dtype=dtype, device=DEV)
+        self.v_pages = torch.zeros(n_pages, n_kv, head_dim, page_size, dtype=dtype, device=DEV)
+        g = torch.Generator().manual_seed(seed)
+        perm = torch.randperm(n_pages, generator=g).tolist()  # pages in no particular order
+        width = max(-(-kv // page_size) for kv in kv_lens)
+        table = torch.full((len(kv_lens), width), -1, dtype=torch.int32)
+        for s, kv in enumerate(kv_lens):
+            for i in range(-(-kv // page_size)):
+                table[s, i] = perm.pop()
+        self.block_table = table.to(DEV)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [72, 1000, 3072])
+def test_embed(hip, dtype, hidden):
+    table = rnd(517, hidden, dtype=dtype)
+    ids = torch.tensor([0, 516, 3, 3, 100], dtype=torch.int32, device=DEV)
+    assert torch.equal(hip.embed(ids, table), twin.embed(ids, table))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [40, 1000, 3072, 5000])
+def test_add_rmsnorm(hip, dtype, hidden):
+    res = rnd(7, hidden, seed=1, scale=3.0)
+    delta = rnd(7, hidden, dtype=dtype, seed=2)
+    w = 1 + 0.1 * rnd(hidden, seed=3)
+    r1, r2 = res.clone(), res.clone()
+    out = hip.add_rmsnorm(r1, delta, w, 1e-5, dtype)
+    ref = twin.add_rmsnorm(r2, delta, w, 1e-5, dtype)
+    torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+    torch.testing.assert_close(r1, r2, rtol=0, atol=0)
+    # no delta; selected rows leave the residual alone
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    r3 = res.clone()
+    out = hip.add_rmsnorm(r3, delta, w, 1e-5, dtype, rows)
+    ref = twin.add_rmsnorm(res.clone(), delta, w, 1e-5, dtype, rows)
+    torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+    assert torch.equal(r3, res)
+    out = hip.add_rmsnorm(r3, None, w, 1e-5, dtype)
+    torch.testing.assert_close(out.float(), twin.add_rmsnorm(res.clone(), None, w, 1e-5, dtype).float(), **tol(dtype))
+
+
+def test_rmsnorm_eps_is_inside_the_root(hip):
+    x = torch.full((1, 64), 1e-4, device=DEV)
+    w = torch.ones(64, device=DEV)
+    out = hip.add_rmsnorm(x.clone(), None, w, 1e-2, torch.float32)
+    assert abs(out[0, 0].item() - 1e-4 / math.sqrt(1e-8 + 1e-2)) < 1e-8
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("inter", [24, 1000, 8192])
+def test_swiglu(hip, dtype, inter):
+    gu = rnd(5, 2 * inter, dtype=dtype, scale=3.0)
+    torch.testing.assert_close(hip.swiglu(gu).float(), twin.swiglu(gu).float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(1, 37, 50), (5, 130, 77), (70, 64, 256), (130, 3, 1000)])
+def test_gemm_generic(hip, dtype, shape):
+    M, N, K = shape
+    x, w = rnd(M, K, dtype=dtype, seed=1), rnd(N, K, dtype=dtype, seed=2)
+    ref = x.double() @ w.double().T
+    out = hip.gemm_generic(x, w, out_float32=True)
+    torch.testing.assert_close(out.double(), ref, rtol=1e-5, atol=1e-4)
+    if dtype == torch.bfloat16:
+        out = hip.gemm_generic(x, w)
+        assert out.dtype == torch.bfloat16
+        torch.testing.assert_close(out.double(), ref, rtol=1e-2, atol=1e-2)
+
+
+def test_float32_product_has_no_reduced_precision(hip):
+    """An operand bit below bfloat16 (8 bits) and tf32 (10 bits) resolution must reach the product."""
+    K = 8
+    x = torch.ones(1, K, device=DEV)
+    w = torch.ones(2, K, device=DEV)
+    w[1, 3] += 2.0 ** -12
+    y = hip.linear(x, w)
+    assert y.dtype == torch.float32
+    assert y[0, 0].item() == 8.0
+    assert y[0, 1].item() - 8.0 == 2.0 ** -12
+
+
+def test_linear_rows_do_not_depend_on_the_batch(hip):
+    x, w = rnd(67, 300, seed=1), rnd(130, 300, seed=2)
+    whole = hip.linear(x, w)
+    assert torch.equal(whole[13:14], hip.linear(x[13:14].contiguous(), w))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geom", [
+    # heads, kv heads, head_dim, rotary_dim, page_size
+    (4, 2, 16, 16, 4), (3, 1, 32, 32, 8), (6, 3, 80, 80, 16), (8, 8, 128, 64, 32), (2, 1, 256, 256, 64),
+    (5, 5, 48, 0, 2),
+])
+def test_rope_kv_write_and_attention(hip, dtype, geom):
+    n_heads, n_kv, D, rd, ps = geom
+    q_lens, kv_lens = [1, 7, 64, 3], [130, 7, 64 + 37, 66]
+    ctx = Ctx(q_lens, kv_lens)
+    pages = sum(-(-kv // ps) for kv in kv_lens) + 3
+    c_hip = Cache(pages, n_kv, ps, D, dtype, kv_lens, seed=4)
+    c_twin = Cache(pages, n_kv, ps, D, dtype, kv_lens, seed=4)
+    # earlier tokens' keys and values already in the pages (same in both)
+    c_hip.k_pages.copy_(rnd(*c_hip.k_pages.shape, dtype=dtype, seed=5)); c_twin.k_pages.copy_(c_hip.k_pages)
+    c_hip.v_pages.copy_(rnd(*c_hip.v_pages.shape, dtype=dtype, seed=6)); c_twin.v_pages.copy_(c_hip.v_pages)
+    qkv = rnd(ctx.n_tokens, (n_heads + 2 * n_kv) * D, dtype=dtype, seed=7)
+    q1, q2 = qkv.clone(), qkv.clone()
+    pos = torch.arange(256, dtype=torch.float32)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, max(rd, 2), 2, dtype=torch.float32) / max(rd, 2)))
+    ang = torch.outer(pos, inv)
+    cos, sin = ang.cos().to(DEV), ang.sin().to(DEV)
+    hip.rope_kv_write(q1, n_heads, n_kv, D, rd, cos, sin, ctx, c_hip)
+    twin.rope_kv_write(q2, n_heads, n_kv, D, rd, cos, sin, ctx, c_twin)
+    torch.testing.assert_close(q1.float(), q2.float(), **tol(dtype))
+    torch.testing.assert_close(c_hip.k_pages.float(), c_twin.k_pages.float(), **tol(dtype))
+    assert torch.equal(c_hip.v_pages, c_twin.v_pages)
+    for window in (None, 19):
+        out = hip.paged_attention(q2, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, c_twin)
+        ref = twin.paged_attention(q2, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, c_twin)
+        torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
+def test_attention_finds_a_far_key(hip):
+    """One key among hundreds is made to stand out; the output must be its value row."""
+    n_heads, n_kv, D, ps = 2, 1, 64, 16
+    kv = 700
+    ctx = Ctx([1], [kv])
+    cache = Cache(64, n_kv, ps, D, torch.float32, [kv])
+    cache.k_pages.copy_(0.01 * rnd(*cache.k_pages.shape, seed=1))
+    cache.v_pages.copy_(rnd(*cache.v_pages.shape, seed=2))
+    far = 37
+    page = int(cache.block_table[0, far // ps])
+    direction = torch.nn.functional.normalize(rnd(D, seed=3), dim=0)
+    cache.k_pages[page, 0, far % ps] = 40.0 * direction
+    qkv = torch.zeros(1, (n_heads + 2 * n_kv) * D, device=DEV)
+    qkv[0, :D] = 40.0 * direction
+    qkv[0, D:2 * D] = 40.0 * direction
+    out = hip.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), None, ctx, cache)
+    want = cache.v_pages[page, 0, :, far % ps]
+    torch.testing.assert_close(out[0, :D], want, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(out[0, D:], want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("vocab", [16, 1000, 128256])
+def test_sample_matches_twin(hip, vocab):
+    rows = 12
+    logits = rnd(rows, vocab, seed=1, scale=2.0)
+    temperature = torch.tensor([0, 0, 1, 1, 0.7, 0.7, 1.3, 1, 1, 0.5, 1, 2], dtype=torch.float32, device=DEV)
+    top_k = torch.tensor([0, 5, 0, 0, 5, 0, 50, 1, 0, 3, vocab, 7], dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([1, 1, 1, 1, 1, 0.9, 0.5, 1, 0.0, 0.8, 1, 0.3], dtype=torch.float32, device=DEV)
+    for seed in range(4):
+        u = torch.rand(rows, generator=torch.Generator().manual_seed(seed)).to(DEV)
+        got = hip.sample(logits, temperature, top_k, top_p, u)
+        ref = twin.sample(logits, temperature, top_k, top_p, u)
+        assert got.tolist() == ref.tolist(), (seed, got.tolist(), ref.tolist())
+
+
+def test_sample_greedy_is_argmax_with_lowest_index_on_ties(hip):
+    logits = torch.zeros(3, 5000, device=DEV)
+    logits[0, 4321] = 1.0
+    logits[1, [17, 4000]] = 2.0
+    z = lambda dt, v: torch.full((3,), v, dtype=dt, device=DEV)
+    got = hip.sample(logits, z(torch.float32, 0.0), z(torch.int32, 0), z(torch.float32, 1.0), z(torch.float32, 0.5))
+    assert got.tolist() == [4321, 17, 0]

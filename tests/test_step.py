@@ -1,0 +1,173 @@
+"""The step function against the plain implementation, under every way of cutting the work.
+
+The same tests run on the CPU with the torch twins of the kernels (marked not gpu: they
+test the cache manager and the batch layout) and on the GPU with the HIP kernels in float32
+and in bfloat16 (marked gpu).
+"""
+
+import pytest
+import torch
+
+from helpers import TINIES, TOLERANCE, make_runner, plain_logits, random_tokens, rel_err, write_tiny_model
+from simple_inference_amd.engine import StepEntry
+
+BACKENDS = [
+    pytest.param("twins"),
+    pytest.param("hip-f32", marks=pytest.mark.gpu),
+    pytest.param("hip-bf16", marks=pytest.mark.gpu),
+]
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name, tiny in TINIES.items():
+        out[name] = write_tiny_model(tmp_path_factory.mktemp(f"tiny_{name}"), tiny, seed=11 + len(name))
+    return out
+
+
+def replay(runner, cache, schedule):
+    """schedule: list of steps; a step is (entries, ends); an entry is (req, tokens, want).
+    Returns {req: {position: logits row}}."""
+    got = {}
+    fed = {}
+    for entries, ends in schedule:
+        step_entries = []
+        for req, tokens, want in entries:
+            if req not in cache.lengths:
+                cache.admit(req)
+                fed[req] = 0
+            step_entries.append(StepEntry(req, tokens, want))
+        logits = runner.run(step_entries)
+        r = 0
+        for req, tokens, want in entries:
+            for w in want:
+                got.setdefault(req, {})[fed[req] + w] = logits[r].float().cpu()
+                r += 1
+            fed[req] += len(tokens)
+        for req in ends:
+            cache.release(req)
+        cache.check()
+    return got
+
+
+def check_against_plain(got, prompts, folder, backend):
+    worst = 0.0
+    for req, rows in got.items():
+        ref = plain_logits(folder, prompts[req])
+        pos = sorted(rows)
+        mine = torch.stack([rows[p] for p in pos])
+        worst = max(worst, rel_err(mine, ref[pos]))
+    assert worst <= TOLERANCE[backend], f"worst relative difference {worst:.3e} > {TOLERANCE[backend]:.1e}"
+    return worst
+
+
+def cut(tokens, sizes):
+    """Cuts a token list into portions whose sizes cycle through ``sizes``."""
+    out, i, k = [], 0, 0
+    while i < len(tokens):
+        n = min(sizes[k % len(sizes)], len(tokens) - i)
+        out.append(tokens[i:i + n])
+        i += n
+        k += 1
+    return out
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", list(TINIES))
+def test_whole_prompts_alone(folders, backend, name):
+    tiny = TINIES[name]
+    runner, cache, mcfg = make_runner(folders[name], backend, tiny.page_size, num_pages=64)
+    prompts = {i: random_tokens(mcfg.vocab_size, n, seed=i) for i, n in enumerate((1, 5, 17, 70, 131))}
+    schedule = [([(r, t, list(range(len(t))))], [r]) for r, t in prompts.items()]
+    got = replay(runner, cache, schedule)
+    check_against_plain(got, prompts, folders[name], backend)
+    assert all(cache.free_pages(g) == 64 for g in range(len(cache.groups)))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", list(TINIES))
+def test_last_32_tokens_one_by_one(folders, backend, name):
+    tiny = TINIES[name]
+    runner, cache, mcfg = make_runner(folders[name], backend, tiny.page_size, num_pages=64)
+    tokens = random_tokens(mcfg.vocab_size, 97, seed=5)
+    head = len(tokens) - 32
+    schedule = [([(0, tokens[:head], [head - 1])], [])]
+    schedule += [([(0, [tokens[i]], [0])], []) for i in range(head, len(tokens))]
+    got = replay(runner, cache, schedule)
+    assert sorted(got[0]) == list(range(head - 1, len(tokens)))
+    check_against_plain(got, {0: tokens}, folders[name], backend)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", list(TINIES))
+def test_portions_of_changing_size(folders, backend, name):
+    tiny = TINIES[name]
+    runner, cache, mcfg = make_runner(folders[name], backend, tiny.page_size, num_pages=64)
+    tokens = random_tokens(mcfg.vocab_size, 150, seed=6)
+    schedule = [([(0, part, list(range(len(part))))], []) for part in cut(tokens, [2, 7, 3, 16, 2, 33, 5, 64, 9])]
+    got = replay(runner, cache, schedule)
+    check_against_plain(got, {0: tokens}, folders[name], backend)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", list(TINIES))
+def test_mixed_requests_with_page_reuse(folders, backend, name):
+    """Up to four live requests; portions of some beside single tokens of others; the pool is so
+    small that pages of finished requests are handed out again."""
+    tiny = TINIES[name]
+    ps = tiny.page_size
+    lengths = [70, 45, 90, 33, 64, 51, 80]
+    vocab = tiny.config["vocab_size"]
+    prompts = {i: random_tokens(vocab, n, seed=100 + i) for i, n in enumerate(lengths)}
+    # four largest live at once, each rounded up to whole pages
+    pool = sum(sorted(-(-n // ps) for n in lengths)[-4:])
+    runner, cache, mcfg = make_runner(folders[name], backend, ps, num_pages=pool)
+
+    # every request: a first portion, then portions of changing size, its last 6 tokens one by one
+    plans = {}
+    for r, toks in prompts.items():
+        body, tail = toks[:-6], toks[-6:]
+        plans[r] = cut(body, [11 + r, 2, 5, 23]) + [[t] for t in tail]
+    waiting = list(prompts)
+    live, schedule, pages_seen = [], [], set()
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries, ends = [], []
+        for r in list(live):
+            if (len(schedule) + r) % 5 == 4 and len(live) > 1:
+                continue  # a request may be left out of a step and go on later
+            part = plans[r].pop(0)
+            entries.append((r, part, list(range(len(part)))))
+            if not plans[r]:
+                ends.append(r)
+                live.remove(r)
+        schedule.append((entries, ends))
+    assert any(len(e) == 4 for e, _ in schedule)
+    got = replay(runner, cache, schedule)
+    check_against_plain(got, prompts, folders[name], backend)
+    assert all(cache.free_pages(g) == pool for g in range(len(cache.groups)))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_first_tokens_of_a_sequence(folders, backend):
+    """Position 0 sees one key; its logits are those of a one-token sequence."""
+    tiny = TINIES["b"]
+    runner, cache, mcfg = make_runner(folders["b"], backend, tiny.page_size, num_pages=16)
+    tokens = random_tokens(mcfg.vocab_size, 3, seed=9)
+    got = replay(runner, cache, [([(0, [tokens[0]], [0])], []), ([(0, [tokens[1]], [0])], []),
+                                 ([(0, [tokens[2]], [0])], [0])])
+    check_against_plain(got, {0: tokens}, folders["b"], backend)
+    one = plain_logits(folders["b"], tokens[:1])
+    assert rel_err(got[0][0][None], one) <= TOLERANCE[backend]
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_long_decoding(folders, backend):
+    tiny = TINIES["a"]
+    runner, cache, mcfg = make_runner(folders["a"], backend, tiny.page_size, num_pages=128)
+    tokens = random_tokens(mcfg.vocab_size, 300, seed=10)
+    schedule = [([(0, tokens[:4], [3])], [])] + [([(0, [t], [0])], []) for t in tokens[4:]]
+    got = replay(runner, cache, schedule)
+    check_against_plain(got, {0: tokens}, folders["a"], backend)
