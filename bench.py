@@ -1,0 +1,182 @@
+"""Measurement: decode tokens a second and prefill tokens a second at the Llama-3.2-3B shape.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  A "step" is one decode step of the engine (scheduler, one call of the
+step function over the batch, sampling).  The default run has the layer sizes of the 3B shape
+(28 layers, hidden 3072, 24 query / 8 key-value heads of 128, feed-forward 8192, vocabulary
+128256, tied head) with seeded random bfloat16 weights, a batch of 8 requests, each with a
+2,048-token context of uniform-random token ids, and a context limit of 4,096.  Beside the
+headline it reports the prefill of one 2,048-token prompt, decode at batch 1 and 64, and how
+close the decode step comes to the HBM roofline and the prefill to the matrix-core peak.
+
+The engine runs on one GPU; asked for more it says so and exits with 2.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+import torch
+
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, published
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}   # dense matrix-core peaks, published
+
+
+def parse_args(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=2048, help="tokens each request holds before decoding")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--preset", default="llama-3.2-3b")
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the preset has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--block-size", type=int, default=None)
+    ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--points", default="1,64", help="further decode batch sizes to report, comma separated")
+    ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    return ap.parse_args(argv)
+
+
+def build_engine(args, max_batch, total_len):
+    from simple_inference_amd import Engine, EngineConfig, preset
+
+    cfg = preset(args.preset)
+    layers_full = cfg["num_hidden_layers"]
+    if args.layers is not None:
+        cfg["num_hidden_layers"] = args.layers
+    kw = {}
+    if args.block_size:
+        kw["block_size"] = args.block_size
+    ecfg = EngineConfig(
+        max_running=max_batch, max_seq_len=4096, dtype=args.dtype, chunk_tokens=max(2048, args.prefill_tokens),
+        eos_id=-1, use_graphs=not args.no_graphs, device="cuda:0", **kw)
+    ecfg.num_kv_blocks = max_batch * (-(-total_len // ecfg.block_size)) + 8
+    engine = Engine.from_random(cfg, seed=args.seed, engine_cfg=ecfg, std=0.02, generate_on_device=True)
+    return engine, cfg, layers_full
+
+
+def matmul_params(mc):
+    """Weights of the matrix products of one forward pass of one token (head included once)."""
+    q = mc.num_attention_heads * mc.head_dim
+    kv = mc.num_key_value_heads * mc.head_dim
+    per_layer = mc.hidden_size * (q + 2 * kv) + q * mc.hidden_size + 3 * mc.hidden_size * mc.intermediate_size
+    return mc.num_hidden_layers * per_layer, mc.vocab_size * mc.hidden_size
+
+
+def random_prompt(vocab, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def measure_decode(engine, batch, context, steps, warmup, seed=0):
+    """(seconds per step, mean context over the timed steps) with ``batch`` requests decoding."""
+    from simple_inference_amd import SamplingParams
+
+    engine.reset()
+    vocab = engine.model.vocab_size
+    params = SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + batch + 2, ignore_eos=True)
+    reqs = [engine.add_request(random_prompt(vocab, context, seed + i), params=params) for i in range(batch)]
+    while any(r.num_generated == 0 for r in reqs):   # prefill every prompt
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    ctx0 = sum(r.context_len for r in reqs) / batch
+    before = [r.num_generated for r in reqs]
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    ctx1 = sum(r.context_len for r in reqs) / batch
+    assert all(r.num_generated == b + steps for r, b in zip(reqs, before)), "a request did not decode in every step"
+    engine.reset()
+    return dt, (ctx0 + ctx1) / 2
+
+
+def measure_prefill(engine, tokens, repeats=3, seed=100):
+    from simple_inference_amd import SamplingParams
+
+    vocab = engine.model.vocab_size
+    best = None
+    for i in range(repeats + 1):   # the first is warmup
+        engine.reset()
+        engine.add_request(random_prompt(vocab, tokens, seed + i), params=SamplingParams(max_new_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if i > 0:
+            best = dt if best is None else min(best, dt)
+    engine.reset()
+    return best
+
+
+def main(argv=None):
+    args = parse_args(argv)
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    points = [int(p) for p in args.points.split(",") if p]
+    max_batch = max([args.batch] + points)
+    total_len = max(args.context + args.warmup + args.steps + max_batch + 2, args.prefill_tokens + 2)
+    engine, cfg, layers_full = build_engine(args, max_batch, total_len)
+    mc = engine.model_cfg
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    el = 2 if args.dtype == "bfloat16" else 4
+    layer_w, head_w = matmul_params(mc)
+
+    def decode_point(batch):
+        dt, ctx = measure_decode(engine, batch, args.context, args.steps, args.warmup, args.seed)
+        bytes_read = (layer_w + head_w) * el + batch * ctx * mc.kv_bytes_per_token(el)
+        return dt, batch / dt, bytes_read / dt / 1e9
+
+    dt, tok_s, gbs = decode_point(args.batch)
+    line = {
+        "metric": "decode tok/s at batch 8; prefill tok/s at 2,048 tokens (3B, bf16)"
+                  if args.batch == 8 else f"decode tok/s at batch {args.batch}",
+        "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dt_name, "data": "synthetic (seeded random weights N(0, 0.02) and uniform-random token ids)",
+        "config": {
+            "model": args.preset + "-shape", "layers": mc.num_hidden_layers, "layers_full": layers_full,
+            "hidden": mc.hidden_size, "heads": mc.num_attention_heads, "kv_heads": mc.num_key_value_heads,
+            "head_dim": mc.head_dim, "intermediate": mc.intermediate_size, "vocab": mc.vocab_size,
+            "global_batch": args.batch, "seq_len": args.context, "context_limit": 4096,
+            "page_size": engine.cfg.block_size, "graphs": engine.graphs is not None, "parallelism": "single GPU",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / PEAK_HBM_GBS, 4)},
+    }
+    if not args.no_prefill:
+        T = args.prefill_tokens
+        sec = measure_prefill(engine, T)
+        attn_flops = mc.num_hidden_layers * 4 * mc.num_attention_heads * mc.head_dim * T * (T + 1) / 2
+        flops = 2 * layer_w * T + 2 * head_w * 1 + attn_flops
+        line["prefill"] = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
+                           "frac": round(flops / sec / PEAK_FLOPS[dt_name], 4)}
+    pts = {}
+    for b in points:
+        _, p_tok_s, p_gbs = decode_point(b)
+        pts[f"decode_b{b}"] = round(p_tok_s, 2)
+        pts[f"decode_b{b}_hbm_frac"] = round(p_gbs / PEAK_HBM_GBS, 4)
+    if pts:
+        line["points"] = pts
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

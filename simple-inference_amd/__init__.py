@@ -2,5 +2,8 @@
 
 from . import models  # noqa: F401  (registers the architectures)
 from .config import EngineConfig, LlamaConfig, preset, register_architecture
+from .engine import Engine, Request, RequestState
+from .sampling import SamplingParams
 
-__all__ = ["EngineConfig", "LlamaConfig", "preset", "register_architecture"]
+__all__ = ["EngineConfig", "LlamaConfig", "preset", "register_architecture", "Engine", "Request",
+           "RequestState", "SamplingParams"]

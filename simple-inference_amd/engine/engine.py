@@ -1,0 +1,260 @@
+"""The engine: requests in, tokens out (reference: ``serving/engine.py:95-517``).
+
+``add_request`` queues a request; ``step`` runs one iteration: finished requests leave, waiting
+ones are admitted while slots, token budget and pages allow, the scheduler picks this step's
+tokens (one per decoding request, then prompt portions), ONE call of the step function runs
+them all as one batch, and the sampler turns the returned logits into tokens.  ``run`` steps
+until nothing is left.  The reference's step runs two forwards instead, one for whole prompts
+and one for decoded tokens (``serving/engine.py:330-349``).
+"""
+
+from __future__ import annotations
+
+import time
+from typing import Dict, Iterator, List, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..config.engine_config import EngineConfig
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from .build import default_kernels, model_from_folder, model_from_random
+from .request import Request, RequestState
+from .scheduler import Scheduler
+from .step import StepEntry, StepRunner
+
+
+class Engine:
+    def __init__(self, model, model_cfg, engine_cfg: EngineConfig, kernels):
+        self.model = model
+        self.model_cfg = model_cfg
+        self.cfg = engine_cfg
+        self.kernels = kernels
+        self.device = torch.device(engine_cfg.device)
+        self.max_seq_len = engine_cfg.max_seq_len
+        plan = model.plan
+        if engine_cfg.eos_id is None:
+            self.eos_ids = tuple(plan.eos_token_ids)
+        elif engine_cfg.eos_id < 0:
+            self.eos_ids = ()
+        else:
+            self.eos_ids = (engine_cfg.eos_id,)
+        self.cache = CacheManager(
+            model.cache_layout(), page_size=engine_cfg.block_size, num_pages=engine_cfg.resolved_num_kv_blocks(),
+            max_running=engine_cfg.max_running, dtype=engine_cfg.torch_dtype, device=self.device)
+        self.runner = StepRunner(model, self.cache, kernels, self.device, engine_cfg.max_seq_len)
+        self.scheduler = Scheduler(engine_cfg.max_running, engine_cfg.resolved_token_budget(),
+                                   engine_cfg.chunk_tokens)
+        self.sampler = Sampler(kernels, self.device)
+        self.prefix_cache = None
+        if engine_cfg.use_prefix_cache:
+            from ..cache.prefix import PrefixCache
+            cap = engine_cfg.prefix_cache_blocks or engine_cfg.resolved_num_kv_blocks()
+            self.prefix_cache = PrefixCache(self.cache, max_pages=cap)
+        self.graphs = None
+        if engine_cfg.use_graphs:
+            from .graphs import GraphedDecode
+            self.graphs = GraphedDecode(self)
+        self.stats = {"steps": 0, "tokens_run": 0, "prefill_tokens": 0, "decode_tokens": 0}
+        if engine_cfg.warmup:
+            self.warmup()
+
+    # -- construction ----------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder, engine_cfg: Optional[EngineConfig] = None, kernels=None) -> "Engine":
+        engine_cfg = engine_cfg or EngineConfig()
+        kernels = kernels if kernels is not None else default_kernels()
+        model, model_cfg = model_from_folder(folder, engine_cfg, kernels)
+        return cls(model, model_cfg, engine_cfg, kernels)
+
+    @classmethod
+    def from_random(cls, config_dict, seed: int = 0, engine_cfg: Optional[EngineConfig] = None, kernels=None,
+                    **random_options) -> "Engine":
+        engine_cfg = engine_cfg or EngineConfig()
+        kernels = kernels if kernels is not None else default_kernels()
+        model, model_cfg = model_from_random(config_dict, seed, engine_cfg, kernels, **random_options)
+        return cls(model, model_cfg, engine_cfg, kernels)
+
+    # -- requests ----------------------------------------------------------------
+    def add_request(self, prompt_tokens: Sequence[int], max_new_tokens: Optional[int] = None,
+                    params: Optional[SamplingParams] = None) -> Request:
+        """Queues a request (reference: ``serving/engine.py:228-254``, same checks)."""
+        prompt = [int(t) for t in prompt_tokens]
+        if params is None:
+            params = SamplingParams(max_new_tokens=max_new_tokens if max_new_tokens is not None else 16)
+        elif max_new_tokens is not None:
+            params = SamplingParams(**{**params.__dict__, "max_new_tokens": max_new_tokens})
+        if not prompt:
+            raise ValueError("prompt_tokens is empty")
+        total = len(prompt) + params.max_new_tokens
+        if total > self.max_seq_len:
+            raise ValueError(f"prompt_len ({len(prompt)}) + max_new_tokens ({params.max_new_tokens}) "
+                             f"> max_seq_len ({self.max_seq_len})")
+        for g in self.cache.groups:
+            need = g.pages_to_reserve(total, self.cfg.chunk_tokens)
+            if need > g.num_pages:
+                raise ValueError(f"request needs more pages than the whole cache: {need} > {g.num_pages}")
+        vocab = self.model.vocab_size
+        if any(t < 0 or t >= vocab for t in prompt):
+            raise ValueError("prompt contains out-of-range token ids")
+        req = Request(prompt_tokens=prompt, params=params)
+        self.scheduler.add(req)
+        return req
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    def reset(self) -> None:
+        """Drops every request and gives every page and slot back."""
+        self.scheduler.waiting.clear()
+        self.scheduler.running.clear()
+        self.cache.reset()
+        if self.prefix_cache is not None:
+            self.prefix_cache.clear()
+
+    # -- admission ----------------------------------------------------------------
+    def _try_admit(self, req: Request) -> bool:
+        total = req.prompt_len + req.max_new_tokens
+        shared: List[int] = []
+        if self.prefix_cache is not None:
+            shared = self.prefix_cache.match(req.prompt_tokens)
+            need = self.cache.groups[0].pages_to_reserve(total, self.cfg.chunk_tokens) - len(shared)
+            if not self.prefix_cache.evict_until_available(need, protected=set(shared)):
+                return False
+        if not self.cache.can_admit(total, self.cfg.chunk_tokens, len(shared)):
+            return False
+        req.slot = self.cache.admit(req.id, total, self.cfg.chunk_tokens, shared_pages=shared)
+        req.cached_prefix_len = len(shared) * self.cfg.block_size
+        req.num_computed = req.cached_prefix_len
+        return True
+
+    # -- one iteration ---------------------------------------------------------------
+    @torch.no_grad()
+    def step(self) -> Dict[int, int]:
+        """Runs one iteration; returns {request id: token} for every request that emitted one."""
+        self.scheduler.evict_finished()
+        self.scheduler.admit(self._try_admit)
+        plan = self.scheduler.plan_step()
+        if not plan:
+            return {}
+        entries, emitters = [], []
+        for req, n in plan:
+            if req.state is RequestState.DECODE:
+                entries.append(StepEntry(req.id, [req.last_token], [0]))
+                emitters.append(req)
+                self.stats["decode_tokens"] += 1
+            else:
+                tokens = req.prompt_tokens[req.num_computed:req.num_computed + n]
+                last = req.num_computed + n == req.prompt_len
+                entries.append(StepEntry(req.id, tokens, [n - 1] if last else []))
+                if last:
+                    emitters.append(req)
+                self.stats["prefill_tokens"] += n
+        self.stats["steps"] += 1
+        self.stats["tokens_run"] += sum(n for _, n in plan)
+
+        if self.graphs is not None and self.graphs.can_run(plan):
+            logits = self.graphs.run(entries)
+        else:
+            logits = self.runner.run(entries)
+        for req, n in plan:
+            req.num_computed += n
+        emitted: Dict[int, int] = {}
+        if emitters:
+            tokens = self.sampler.sample(logits, [r.params for r in emitters], [r.num_generated for r in emitters])
+            for req, token in zip(emitters, tokens):
+                self._emit(req, int(token))
+                emitted[req.id] = int(token)
+        return emitted
+
+    def _emit(self, req: Request, token: int) -> None:
+        """Appends a token and moves the request on (reference: ``serving/engine.py:449-460,499-507``)."""
+        if req.state is RequestState.PREFILL and self.prefix_cache is not None:
+            self.prefix_cache.insert(req.prompt_tokens, self.cache.table(0, req.id))
+        req.generated.append(token)
+        if token in self.eos_ids and not req.params.ignore_eos:
+            req.eos_hit = True
+        if req.should_finish():
+            req.state = RequestState.FINISHED
+            self.cache.release(req.id)   # pages and slot go back at once; the next step may hand them out
+            req.slot = None
+        else:
+            req.state = RequestState.DECODE
+
+    def run(self) -> Dict[int, Request]:
+        """Steps until every queued request has finished; returns them by id."""
+        seen: Dict[int, Request] = {r.id: r for r in self.scheduler.waiting}
+        seen.update({r.id: r for r in self.scheduler.running})
+        while self.has_work():
+            self.step()
+            for r in self.scheduler.running:
+                seen[r.id] = r
+        return seen
+
+    def warmup(self, num_seqs: int = 2, prompt_len: int = 8, decode_steps: int = 4) -> None:
+        """Runs dummy requests through prefill and decode, then resets (reference: ``serving/engine.py:277-312``)."""
+        num_seqs = max(1, min(num_seqs, self.cfg.max_running))
+        prompt_len = max(1, min(prompt_len, self.max_seq_len - decode_steps - 1))
+        vocab = self.model.vocab_size
+        dummy = [i % vocab for i in range(prompt_len)]
+        for _ in range(num_seqs):
+            self.add_request(dummy, params=SamplingParams(max_new_tokens=decode_steps + 1, ignore_eos=True))
+        guard = prompt_len + decode_steps + num_seqs + 8
+        while self.has_work() and guard > 0:
+            self.step()
+            guard -= 1
+        if self.graphs is not None:
+            self.graphs.capture_all()
+        if self.device.type == "cuda":
+            torch.cuda.synchronize(self.device)
+        self.reset()
+
+    # -- single-stream entry points ------------------------------------------------------
+    def generate(self, prompt_tokens: Sequence[int], max_new_tokens: int = 256, temperature: float = 1.0,
+                 top_k: int = 50, top_p: float = 0.9, seed: int = 0) -> Iterator[int]:
+        """Yields the tokens of one request as they come; stops at EOS without yielding it
+        (reference: ``generate.py:50-119``, same option names and defaults)."""
+        req = self.add_request(prompt_tokens, params=SamplingParams(
+            temperature=temperature, top_k=top_k, top_p=top_p, seed=seed, max_new_tokens=max_new_tokens))
+        sent = 0
+        while req.state is not RequestState.FINISHED:
+            self.step()
+            while sent < len(req.generated):
+                token = req.generated[sent]
+                sent += 1
+                if req.eos_hit and sent == len(req.generated):
+                    return
+                yield token
+
+    def generate_with_stats(self, prompt_tokens: Sequence[int], max_new_tokens: int = 256, temperature: float = 1.0,
+                            top_k: int = 50, top_p: float = 0.9, seed: int = 0, on_token=None):
+        """(tokens, stats) with the reference's stat names (``generate.py:227-237``)."""
+        sync = (lambda: torch.cuda.synchronize(self.device)) if self.device.type == "cuda" else (lambda: None)
+        if self.device.type == "cuda":
+            torch.cuda.reset_peak_memory_stats(self.device)
+        sync()
+        t0 = time.perf_counter()
+        t_first = None
+        out: List[int] = []
+        for token in self.generate(prompt_tokens, max_new_tokens, temperature, top_k, top_p, seed):
+            if t_first is None:
+                sync()
+                t_first = time.perf_counter()
+            out.append(token)
+            if on_token is not None:
+                on_token(token)
+        sync()
+        t1 = time.perf_counter()
+        t_first = t_first if t_first is not None else t1
+        n = len(out)
+        decode_s = t1 - t_first
+        stats = {
+            "prompt_tokens": len(prompt_tokens), "new_tokens": n,
+            "ttft_ms": (t_first - t0) * 1e3, "prefill_ms": (t_first - t0) * 1e3,
+            "tpot_ms": decode_s * 1e3 / max(n - 1, 1),
+            "decode_tok_s": (n - 1) / decode_s if n > 1 and decode_s > 0 else 0.0,
+            "total_wall_ms": (t1 - t0) * 1e3, "total_tok_s": n / (t1 - t0) if t1 > t0 else 0.0,
+            "peak_vram_gb": torch.cuda.max_memory_allocated(self.device) / 1e9 if self.device.type == "cuda" else 0.0,
+        }
+        return out, stats
