@@ -66,12 +66,15 @@ class StepRunner:
         self._check(entries)
         cache = self.cache
         n_seqs = len(entries)
-        q_lens = [len(e.tokens) for e in entries]
+        # Sequences that bring one token go first: the kernels treat them apart from longer runs.
+        order = sorted(range(n_seqs), key=lambda i: len(entries[i].tokens) != 1)
+        seqs = [entries[i] for i in order]
+        q_lens = [len(e.tokens) for e in seqs]
+        n_decode = sum(1 for n in q_lens if n == 1)
         n_tokens = sum(q_lens)
-        starts = [cache.extend(e.req, len(e.tokens)) for e in entries]
+        starts = [cache.extend(e.req, len(e.tokens)) for e in seqs]
         n_groups = len(cache.groups)
-        reqs = [e.req for e in entries]
-        width = max(1, cache.max_table_len(reqs))
+        width = max(1, cache.max_table_len([e.req for e in seqs]))
         n_rows = sum(len(e.want) for e in entries)
 
         sizes = [n_tokens, n_tokens, n_tokens, n_seqs + 1, n_seqs, n_seqs, max(n_rows, 1)] + \
@@ -81,23 +84,27 @@ class StepRunner:
         tok, pos, sot, cu, kvl, slots, rows = (host[offsets[i]:offsets[i + 1]] for i in range(7))
         cu[0] = 0
         rows[:] = 0
-        t = r = 0
-        for s, e in enumerate(entries):
+        t = 0
+        first_token = {}
+        for s, e in enumerate(seqs):
             n = q_lens[s]
             tok[t:t + n] = e.tokens
             pos[t:t + n] = np.arange(starts[s], starts[s] + n, dtype=np.int32)
             sot[t:t + n] = s
-            for w in e.want:
-                rows[r] = t + int(w)
-                r += 1
+            first_token[e.req] = t
             t += n
             cu[s + 1] = t
             kvl[s] = starts[s] + n
             slots[s] = cache.slot(e.req)
+        r = 0
+        for e in entries:  # logits come back in the order of the entries as given
+            for w in e.want:
+                rows[r] = first_token[e.req] + int(w)
+                r += 1
         for g in range(n_groups):
             tab = host[offsets[7 + g]:offsets[8 + g]].reshape(n_seqs, width)
             tab[:] = -1
-            for s, e in enumerate(entries):
+            for s, e in enumerate(seqs):
                 row = cache.table(g, e.req)
                 tab[s, :len(row)] = row
 
@@ -108,6 +115,7 @@ class StepRunner:
             token_ids=part(0), positions=part(1), seq_of_token=part(2), cu_q=part(3), kv_len=part(4),
             state_slots=part(5), logit_rows=part(6)[:n_rows] if n_rows else None, n_logit_rows=n_rows,
             max_q_len=max(q_lens), max_kv_len=int(kvl.max()), kernels=self.kernels,
+            n_decode_seqs=n_decode, q_lens=q_lens,
         )
         ctx.block_tables = [part(7 + g).view(n_seqs, width) for g in range(n_groups)]
         return ctx

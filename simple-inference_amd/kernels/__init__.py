@@ -37,6 +37,21 @@ _SIGNATURES = {
 }
 
 
+_ATTN_SIGNATURES = {
+    "sia_attn_decode": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_attn_prefill": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "sia_attn_prefill_rows": [],
+    "sia_attn_mfma_head_dim": [],
+}
+
+
+def attention_library_spec(head_dim: int):
+    """(name, sources, defines) of the matrix-core attention library for one head size."""
+    return (f"attn_mfma_d{head_dim}", ("attention_mfma.hip",), (f"SIA_HEAD_DIM={head_dim}",))
+
+
 class KernelError(RuntimeError):
     pass
 
@@ -63,6 +78,20 @@ class HipKernels:
         self.device = torch.device(device)
         self.core = build.load_library("core")
         _bind(self.core, _SIGNATURES)
+        self._attn_libs = {}
+        self.use_mfma_attention = True   # tests switch it off to reach the plain kernel in bfloat16
+
+    def _attn_lib(self, head_dim: int):
+        """The matrix-core attention kernels for this head size, compiled at first use."""
+        lib = self._attn_libs.get(head_dim)
+        if lib is None:
+            name, sources, defines = attention_library_spec(head_dim)
+            lib = build.load_library(name, sources, defines)
+            _bind(lib, _ATTN_SIGNATURES)
+            if lib.sia_attn_mfma_head_dim() != head_dim:
+                raise KernelError(f"library {name} was built for another head size")
+            self._attn_libs[head_dim] = lib
+        return lib
 
     # -- helpers -------------------------------------------------------------
     def _stream(self):
@@ -228,12 +257,48 @@ class HipKernels:
         self._check_pages(cache.k_pages, cache.v_pages, cache.block_table, cache.page_size, n_kv_heads, head_dim,
                           qkv.dtype, ctx)
         out = torch.empty((n, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+        page = cache.page_size
+        if (self.use_mfma_attention and qkv.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256
+                and page >= 8 and width % 8 == 0):
+            self._mfma_attention(qkv, out, n_heads, n_kv_heads, head_dim, scale, int(window or 0), ctx, cache)
+            return out
         self._check(self.core.sia_attention_generic(
             _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(cache.block_table),
             cache.block_table.shape[1], _ptr(ctx.seq_of_token), _ptr(ctx.positions), _ptr(out), n, n_heads,
-            n_kv_heads, head_dim, cache.page_size, float(scale), int(window or 0), _DT[qkv.dtype],
+            n_kv_heads, head_dim, page, float(scale), int(window or 0), _DT[qkv.dtype],
             self._stream()), "attention_generic")
         return out
+
+    @staticmethod
+    def decode_split(n_seqs: int, n_kv_heads: int, kv_bound: int):
+        """(keys per split, number of splits): the largest split that still gives the chip ~4 waves a CU."""
+        for keys in (512, 256, 128):
+            if n_seqs * n_kv_heads * (-(-kv_bound // keys)) >= 1024:
+                return keys, -(-kv_bound // keys)
+        return 64, -(-kv_bound // 64)
+
+    def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
+        lib = self._attn_lib(head_dim)
+        width = qkv.shape[1]
+        table = cache.block_table
+        n_dec = ctx.n_decode_seqs if n_heads // n_kv_heads <= 16 else 0
+        if n_dec:
+            bound = ctx.kv_bound or ctx.max_kv_len
+            split_keys, max_splits = self.decode_split(n_dec, n_kv_heads, bound)
+            ws_acc = torch.empty((n_dec * n_heads * max_splits * head_dim,), dtype=torch.float32, device=qkv.device)
+            ws_ml = torch.empty((n_dec * n_heads * max_splits * 2,), dtype=torch.float32, device=qkv.device)
+            self._check(lib.sia_attn_decode(
+                _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
+                _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), _ptr(ws_acc), _ptr(ws_ml), n_dec, n_heads,
+                n_kv_heads, cache.page_size, float(scale), window, split_keys, max_splits, self._stream()),
+                "attn_decode")
+        if n_dec < ctx.n_seqs:
+            rows = lib.sia_attn_prefill_rows()
+            n_tiles = sum(-(-q // rows) for q in ctx.q_lens[n_dec:])
+            self._check(lib.sia_attn_prefill(
+                _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
+                _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_heads, n_kv_heads,
+                cache.page_size, float(scale), window, self._stream()), "attn_prefill")
 
     # -- sampling ------------------------------------------------------------------
     def sample(self, logits, temperature, top_k, top_p, uniform):

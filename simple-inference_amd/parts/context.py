@@ -44,6 +44,9 @@ class StepContext:
     max_kv_len: int
     kernels: Any = None
     block_tables: list = field(default_factory=list)  # one [n_seqs, width] table per cache group
+    n_decode_seqs: int = 0  # sequences 0 .. n_decode_seqs-1 bring exactly one token (they are sorted first)
+    q_lens: list = field(default_factory=list)  # host copy: tokens each sequence brings
+    kv_bound: int = 0  # replayed graphs: an upper bound of kv_len that fixes grids (0: use max_kv_len)
 
 
 @dataclass

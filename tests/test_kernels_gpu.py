@@ -44,6 +44,8 @@ class Ctx:
         self.positions, self.seq_of_token, self.cu_q, self.kv_len = i32(pos), i32(sot), i32(cu), i32(kv_lens)
         self.n_tokens, self.n_seqs = len(pos), len(q_lens)
         self.max_q_len, self.max_kv_len = max(q_lens), max(kv_lens)
+        self.q_lens, self.kv_bound = list(q_lens), 0
+        self.n_decode_seqs = next((i for i, q in enumerate(q_lens) if q != 1), len(q_lens))
 
 
 class Cache:
@@ -169,6 +171,34 @@ def test_rope_kv_write_and_attention(hip, dtype, geom):
         out = hip.paged_attention(q2, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, c_twin)
         ref = twin.paged_attention(q2, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, c_twin)
         torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("geom", [
+    # heads, kv heads, head_dim, page_size, window
+    (24, 8, 128, 16, None), (32, 8, 64, 64, None), (16, 1, 32, 8, None), (6, 2, 48, 16, 100), (5, 5, 112, 32, 700),
+    (34, 2, 16, 16, None),
+])
+def test_matrix_core_attention_decode_and_mixed(hip, geom):
+    """Many single-token sequences of different lengths (so that splits differ), alone and beside longer runs."""
+    n_heads, n_kv, D, ps, window = geom
+    dtype = torch.bfloat16
+    for q_lens, kv_lens in (([1] * 7, [1, 63, 64, 65, 300, 1027, 2500]),
+                            ([1, 1, 1, 130, 5, 257], [513, 17, 2048, 130, 900, 300])):
+        ctx = Ctx(q_lens, kv_lens)
+        pages = sum(-(-kv // ps) for kv in kv_lens) + 5
+        cache = Cache(pages, n_kv, ps, D, dtype, kv_lens, seed=8)
+        cache.k_pages.copy_(rnd(*cache.k_pages.shape, dtype=dtype, seed=9))
+        cache.v_pages.copy_(rnd(*cache.v_pages.shape, dtype=dtype, seed=10))
+        qkv = rnd(ctx.n_tokens, (n_heads + 2 * n_kv) * D, dtype=dtype, seed=11)
+        out = hip.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache)
+        ref = twin.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache)
+        torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+        hip.use_mfma_attention = False
+        try:
+            plain_kernel = hip.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache)
+        finally:
+            hip.use_mfma_attention = True
+        torch.testing.assert_close(plain_kernel.float(), ref.float(), **tol(dtype))
 
 
 def test_attention_finds_a_far_key(hip):
