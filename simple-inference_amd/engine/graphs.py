@@ -1,0 +1,177 @@
+"""Decode-only steps replayed from captured hipGraphs.
+
+A decode step launches some nine kernels a layer; at small batches the time to launch them
+exceeds the time they run.  As the reference does with CUDA graphs (``model/cuda_graph.py:62-88``,
+``serving/paged_decoder.py:93-106,260-274``), the whole forward pass of a step in which every
+request brings one token is captured once per batch-size bucket (1, 2, 4, ... up to
+``max_running``) and replayed afterwards.  The rules are the reference's:
+
+* everything a kernel reads that changes from step to step (token ids, positions, lengths, block
+  tables, slots) lives in device buffers of fixed address, filled before each replay; loop bounds
+  come from those buffers, grids from the bucket and the engine's ``max_seq_len``;
+* pages are taken on the host before the replay (``serving/paged_kv_cache.py:258-270``);
+* rows that pad a batch up to its bucket hold token 0 at position 0 and write to the scratch page
+  and scratch slot, which no request owns (``serving/paged_decoder.py:224-247``).
+
+``torch.cuda.CUDAGraph`` is hipGraph on this platform; this package's kernels are launched on
+torch's current stream, so they are captured with the library products between them.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List
+
+import numpy as np
+import torch
+
+from ..parts.context import StepContext
+from .step import StepEntry
+
+
+def buckets_for(max_running: int) -> List[int]:
+    """1, 2, 4, ... and ``max_running`` itself (reference: buckets(7) = [1, 2, 4, 7])."""
+    out, b = [], 1
+    while b < max_running:
+        out.append(b)
+        b *= 2
+    out.append(max_running)
+    return out
+
+
+def kv_buckets_for(max_seq_len: int, smallest: int = 512) -> List[int]:
+    """Bounds on the longest sequence of a step: 512, 1024, ... and ``max_seq_len`` itself.  A graph is
+    captured per bound, so that the attention grid fits the lengths it actually meets."""
+    out, b = [], smallest
+    while b < max_seq_len:
+        out.append(b)
+        b *= 2
+    out.append(max_seq_len)
+    return out
+
+
+class _Bucket:
+    def __init__(self, size, kv_bound, meta, host, offsets, ctx, caches):
+        self.size = size
+        self.kv_bound = kv_bound
+        self.meta = meta          # device int32 buffer, fixed address
+        self.host = host          # host mirror that is filled and copied over
+        self.offsets = offsets
+        self.ctx = ctx
+        self.caches = caches
+        self.graph = None
+        self.logits = None
+
+
+class GraphedDecode:
+    def __init__(self, engine):
+        self.engine = engine
+        self.runner = engine.runner
+        self.cache = engine.cache
+        self.device = engine.device
+        self.max_seq_len = engine.cfg.max_seq_len
+        self.width = engine.cfg.pages_per_request()
+        self.buckets = buckets_for(engine.cfg.max_running)
+        self.kv_buckets = kv_buckets_for(self.max_seq_len)
+        self._made: Dict[tuple, _Bucket] = {}
+        self.replays = 0
+        if self.device.type != "cuda":
+            raise RuntimeError("graph replay needs the GPU")
+
+    # -- which steps ---------------------------------------------------------------
+    def can_run(self, plan) -> bool:
+        return 0 < len(plan) <= self.buckets[-1] and all(n == 1 for _, n in plan)
+
+    def bucket_of(self, rows: int) -> int:
+        return next(b for b in self.buckets if b >= rows)
+
+    # -- buffers ---------------------------------------------------------------------
+    def kv_bucket_of(self, longest: int) -> int:
+        return next(b for b in self.kv_buckets if b >= longest)
+
+    def _make(self, size: int, kv_bound: int) -> _Bucket:
+        n_groups = len(self.cache.groups)
+        sizes = [size, size, size, size + 1, size, size, size] + [size * self.width] * n_groups
+        offsets = [0]
+        for s in sizes:
+            offsets.append(offsets[-1] + s)
+        host = np.zeros(offsets[-1], dtype=np.int32)
+        meta = torch.zeros(offsets[-1], dtype=torch.int32, device=self.device)
+        part = lambda i: meta[offsets[i]:offsets[i + 1]]
+        ctx = StepContext(
+            n_tokens=size, n_seqs=size, token_ids=part(0), positions=part(1), seq_of_token=part(2),
+            cu_q=part(3), kv_len=part(4), state_slots=part(5), logit_rows=part(6), n_logit_rows=size,
+            max_q_len=1, max_kv_len=kv_bound, kernels=self.runner.kernels,
+            n_decode_seqs=size, q_lens=[1] * size, kv_bound=kv_bound)
+        ctx.block_tables = [part(7 + g).view(size, self.width) for g in range(n_groups)]
+        caches = self.cache.layer_caches(ctx.block_tables)
+        return _Bucket(size, kv_bound, meta, host, offsets, ctx, caches)
+
+    def _fill(self, b: _Bucket, entries: List[StepEntry]) -> None:
+        """Takes this step's pages and writes the step's metadata (padding included) into the buffers."""
+        size, off, host = b.size, b.offsets, b.host
+        cache = self.cache
+        tok, pos, sot, cu, kvl, slots, rows = (host[off[i]:off[i + 1]] for i in range(7))
+        tok[:] = 0
+        pos[:] = 0
+        kvl[:] = 1
+        slots[:] = cache.slots.scratch_slot
+        sot[:] = np.arange(size)
+        cu[:] = np.arange(size + 1)
+        rows[:] = np.arange(size)
+        for g, grp in enumerate(cache.groups):
+            host[off[7 + g]:off[8 + g]] = grp.scratch_page
+        for s, e in enumerate(entries):
+            start = cache.extend(e.req, 1)
+            tok[s] = e.tokens[0]
+            pos[s] = start
+            kvl[s] = start + 1
+            slots[s] = cache.slot(e.req)
+            for g in range(len(cache.groups)):
+                row = cache.table(g, e.req)
+                base = off[7 + g] + s * self.width
+                host[base:base + len(row)] = row
+                host[base + len(row):base + self.width] = -1
+        b.meta.copy_(torch.from_numpy(host))
+
+    # -- capture and replay -----------------------------------------------------------
+    @torch.no_grad()
+    def capture(self, size: int, kv_bound: int) -> _Bucket:
+        b = self._make(size, kv_bound)
+        self._fill(b, [])  # padding rows only: they touch the scratch page and slot
+        model = self.runner.model
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                model.forward(b.ctx, b.caches)
+        torch.cuda.current_stream(self.device).wait_stream(side)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            b.logits = model.forward(b.ctx, b.caches)
+        b.graph = graph
+        self._made[(size, kv_bound)] = b
+        return b
+
+    def capture_all(self, kv_bounds=None) -> None:
+        """Captures every batch bucket for the given length bounds (default: the largest only; the
+        others are captured when a step first needs them)."""
+        for kv_bound in (kv_bounds or self.kv_buckets[-1:]):
+            for size in self.buckets:
+                if (size, kv_bound) not in self._made:
+                    self.capture(size, kv_bound)
+
+    @torch.no_grad()
+    def run(self, entries: List[StepEntry]) -> torch.Tensor:
+        self.runner._check(entries)
+        for e in entries:
+            if len(e.tokens) != 1 or list(e.want) != [0]:
+                raise ValueError("a replayed step takes one token per request and returns its logits")
+        size = self.bucket_of(len(entries))
+        longest = max(self.cache.lengths[e.req] for e in entries) + 1
+        kv_bound = self.kv_bucket_of(longest)
+        b = self._made.get((size, kv_bound)) or self.capture(size, kv_bound)
+        self._fill(b, entries)
+        b.graph.replay()
+        self.replays += 1
+        return b.logits[:len(entries)]

@@ -34,6 +34,8 @@ _SIGNATURES = {
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_sample": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "sia_gemm_skinny": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_gemm_skinny_max_rows": [],
 }
 
 
@@ -80,6 +82,8 @@ class HipKernels:
         _bind(self.core, _SIGNATURES)
         self._attn_libs = {}
         self.use_mfma_attention = True   # tests switch it off to reach the plain kernel in bfloat16
+        self.use_skinny_gemm = True      # few-row bfloat16 products by this package's kernel, not the library
+        self._skinny_rows = self.core.sia_gemm_skinny_max_rows()
 
     def _attn_lib(self, head_dim: int):
         """The matrix-core attention kernels for this head size, compiled at first use."""
@@ -156,8 +160,14 @@ class HipKernels:
         M, K = x.shape
         N = w.shape[0]
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+            if (self.use_skinny_gemm and M <= self._skinny_rows and N % 16 == 0 and K % 64 == 0
+                    and (out_float32 or not (N < 4096 and K > 4096))):  # few long rows: the library is faster
+                y = torch.empty((M, N), dtype=torch.float32 if out_float32 else torch.bfloat16, device=x.device)
+                self._check(self.core.sia_gemm_skinny(_ptr(x), _ptr(w), _ptr(y), M, N, K, int(out_float32),
+                                                      self._stream()), "gemm_skinny")
+                return y
             y = torch.mm(x, w.t())  # BLAS library, float accumulation
-            return y.float() if out_float32 else y
+            return self.cast(y, torch.float32) if out_float32 else y
         # True 32-bit product.  A float32-stored matrix meeting bfloat16 activations widens them.
         back = None
         if x.dtype == torch.bfloat16:
@@ -271,17 +281,20 @@ class HipKernels:
 
     @staticmethod
     def decode_split(n_seqs: int, n_kv_heads: int, kv_bound: int):
-        """(keys per split, number of splits): the largest split that still gives the chip ~4 waves a CU."""
-        for keys in (512, 256, 128):
-            if n_seqs * n_kv_heads * (-(-kv_bound // keys)) >= 1024:
+        """(keys per split, number of splits).  A split is one workgroup of four waves, and a compute
+        unit holds two of them: the smallest split whose workgroups all run at once is taken (more,
+        shorter workgroups hide latency better), and 1024 keys when even that many do not."""
+        for keys in (256, 512, 1024):
+            if n_seqs * n_kv_heads * (-(-kv_bound // keys)) <= 512:
                 return keys, -(-kv_bound // keys)
-        return 64, -(-kv_bound // 64)
+        return 1024, -(-kv_bound // 1024)
 
     def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
         lib = self._attn_lib(head_dim)
         width = qkv.shape[1]
         table = cache.block_table
-        n_dec = ctx.n_decode_seqs if n_heads // n_kv_heads <= 16 else 0
+        group = n_heads // n_kv_heads
+        n_dec = ctx.n_decode_seqs if group <= 16 and 4 * group * (head_dim + 2) * 4 <= 65536 else 0
         if n_dec:
             bound = ctx.kv_bound or ctx.max_kv_len
             split_keys, max_splits = self.decode_split(n_dec, n_kv_heads, bound)

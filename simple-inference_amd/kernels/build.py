@@ -36,7 +36,8 @@ HIPCC_FLAGS = [
 # name -> sources.  "core" is everything a model needs in either dtype; further libraries
 # are specialisations compiled for the sizes a model has (see ``specialised``).
 LIBRARIES: Dict[str, Sequence[str]] = {
-    "core": ("elementwise.hip", "rope_cache.hip", "attention_generic.hip", "gemm_generic.hip", "sampling.hip"),
+    "core": ("elementwise.hip", "rope_cache.hip", "attention_generic.hip", "gemm_generic.hip", "gemm_skinny.hip",
+             "sampling.hip"),
 }
 
 

@@ -122,6 +122,28 @@ def test_gemm_generic(hip, dtype, shape):
         torch.testing.assert_close(out.double(), ref, rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("shape", [(1, 48, 64), (8, 5120, 3072), (16, 3072, 8192), (3, 16, 320), (11, 1008, 1024)])
+def test_gemm_skinny(hip, shape):
+    """bfloat16 products with few rows: this package's kernel against a float64 product and the library."""
+    M, N, K = shape
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
+    ref = x.double() @ w.double().T
+    out = hip.linear(x, w, out_float32=True)
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out.double(), ref, rtol=1e-4, atol=1e-3 * math.sqrt(K / 64))
+    out16 = hip.linear(x, w)
+    assert out16.dtype == torch.bfloat16
+    torch.testing.assert_close(out16.double(), ref, rtol=1e-2, atol=1e-2 * math.sqrt(K / 64))
+    hip.use_skinny_gemm = False
+    try:
+        lib = hip.linear(x, w)
+    finally:
+        hip.use_skinny_gemm = True
+    torch.testing.assert_close(out16.float(), lib.float(), rtol=2e-2, atol=2e-2 * math.sqrt(K / 64))
+    # a row's result does not depend on the other rows
+    assert torch.equal(hip.linear(x[:1].contiguous(), w), out16[:1])
+
+
 def test_float32_product_has_no_reduced_precision(hip):
     """An operand bit below bfloat16 (8 bits) and tf32 (10 bits) resolution must reach the product."""
     K = 8
