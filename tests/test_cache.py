@@ -1,0 +1,227 @@
+"""The cache manager: pages, reservations, windows, slots (no GPU)."""
+
+import random
+
+import pytest
+
+from simple_inference_amd.cache import CacheManager, PageAllocator
+from simple_inference_amd.parts.model import CacheLayout
+from simple_inference_amd.parts.plan import PagedKVNeed, StateNeed
+import torch
+
+
+def test_allocator_vector_of_the_reference_test():
+    """serving/test_paged_kv_cache.py:27-43."""
+    a = PageAllocator(4)
+    a.reserve(1, 2)
+    a.reserve(2, 1)
+    assert not a.can_reserve(3, 2)
+    assert (a.allocate(1), a.allocate(1)) == (0, 1)
+    a.share(2, 0)
+    assert a.ref_count(0) == 2
+    a.release(1)
+    assert a.ref_count(0) == 1 and a.free_pages == 3
+    a.release(2)
+    assert a.free_pages == 4
+    a.check()
+
+
+def test_allocator_errors():
+    a = PageAllocator(2)
+    with pytest.raises(KeyError):
+        a.allocate(9)
+    a.reserve(1, 1)
+    with pytest.raises(ValueError):
+        a.can_reserve(1, 1)
+    with pytest.raises(MemoryError):
+        a.reserve(2, 2)
+    p = a.allocate(1)
+    a.reserve(2, 1)
+    with pytest.raises(MemoryError):       # reservation used up and the other page is promised
+        a.allocate(1)
+    with pytest.raises(ValueError):
+        a.share(1, p)
+    with pytest.raises(ValueError):
+        a.share(2, 1)                      # page 1 is free
+    a.free_page(1, p)
+    with pytest.raises(KeyError):          # freed twice
+        a.free_page(1, p)
+    a.release(1), a.release(2), a.release(77)
+    assert a.free_pages == 2
+    a.check()
+
+
+def test_unreserved_allocation_takes_unpromised_pages_only():
+    a = PageAllocator(3)
+    a.reserve(1, 0)
+    a.reserve(2, 2)
+    assert a.allocate(1) == 0              # one page is promised to nobody
+    with pytest.raises(MemoryError):
+        a.allocate(1)
+    assert (a.allocate(2), a.allocate(2)) == (1, 2)
+
+
+def layout(groups, slabs=None, states=()):
+    lay = CacheLayout()
+    lay.kv_groups = list(groups)
+    lay.kv_slabs = list(slabs or [1] * len(groups))
+    lay.run_kv = [(g, 0) for g in range(len(groups))]
+    lay.states = list(states)
+    lay.run_state = [i if i < len(states) else None for i in range(len(groups))]
+    return lay
+
+
+def manager(groups, num_pages=8, page_size=2, max_running=3, states=(), storage=False):
+    return CacheManager(layout(groups, states=states), page_size=page_size, num_pages=num_pages,
+                        max_running=max_running, dtype=torch.float32, device="cpu", allocate_storage=storage)
+
+
+FULL = PagedKVNeed(1, 4)
+
+
+def test_pages_follow_growth_and_come_back_lowest_first():
+    """serving/test_paged_kv_cache.py:58-89: page size 2, 4 pages."""
+    m = manager([FULL], num_pages=4)
+    m.admit(1)
+    assert m.extend(1, 3) == 0 and m.table(0, 1) == [0, 1]
+    assert m.extend(1, 2) == 3 and m.table(0, 1) == [0, 1, 2] and m.lengths[1] == 5
+    m.admit(2)
+    m.extend(2, 1)
+    assert m.table(0, 2) == [3]
+    with pytest.raises(MemoryError):
+        m.extend(2, 2)
+    m.release(1)
+    assert m.free_pages() == 3
+    m.admit(3)
+    m.extend(3, 1)
+    assert m.table(0, 3) == [0]            # the lowest free page is handed out again
+    m.check()
+
+
+def test_reservation_makes_running_out_impossible_in_mid_flight():
+    m = manager([FULL], num_pages=4)
+    assert m.can_admit(8) and not m.can_admit(9)
+    m.admit(1, total_tokens=5)             # 3 pages promised
+    assert not m.can_admit(3) and m.can_admit(2)
+    m.admit(2, total_tokens=2)
+    m.extend(2, 2)
+    m.extend(1, 5)                         # its promised pages are there although request 2 came in between
+    assert sorted(m.table(0, 1) + m.table(0, 2)) == [0, 1, 2, 3]
+    with pytest.raises(MemoryError):
+        m.extend(1, 2)                     # beyond what it declared, and nothing is left
+    m.release(1), m.release(2)
+    assert m.free_pages() == 4 and m.groups[0].allocator.reserved_pages == 0
+
+
+def test_window_group_gives_pages_back_when_the_window_has_passed():
+    win = PagedKVNeed(1, 4, window=4)
+    m = manager([FULL, win], num_pages=16)
+    m.admit(1)
+    pos = 0
+    held = []
+    for n in (3, 2, 1, 1, 6, 1, 1, 1, 1, 1):
+        start = m.extend(1, n)
+        assert start == pos
+        pos += n
+        table = m.table(1, 1)
+        first_visible = max(0, start - 4 + 1)
+        for idx, page in enumerate(table):
+            if idx < first_visible // 2:
+                assert page == -1                          # wholly below the window: given back
+            else:
+                assert page >= 0                           # still visible to this step's first query
+        held.append(sum(p >= 0 for p in table))
+        assert all(p >= 0 for p in m.table(0, 1))          # the full group keeps everything
+        m.check()
+    assert max(held) <= (4 + 6 - 1 + 1) // 2 + 1           # window + largest portion, in pages, plus one
+    assert m.free_pages(1) == 16 - held[-1] and m.free_pages(0) == 16 - len(m.table(0, 1))
+    m.release(1)
+    assert m.free_pages(0) == 16 and m.free_pages(1) == 16
+
+
+def test_window_reservation_is_small_and_sufficient():
+    win = PagedKVNeed(1, 4, window=4)
+    m = manager([win], num_pages=6)
+    g = m.groups[0]
+    assert g.pages_to_reserve(1000, max_chunk=3) == (4 + 3 - 1 + 1) // 2 + 1 == 4
+    assert g.pages_to_reserve(3, max_chunk=3) == 2
+    m.admit(1, total_tokens=1000, max_chunk=3)
+    m.admit(2, total_tokens=3, max_chunk=3)                # 4 + 2 pages promised: the pool is full
+    assert not m.can_admit(1, 1)
+    for _ in range(100):
+        m.extend(1, 3)                                     # never runs out although 300 positions pass
+        m.check()
+    m.extend(2, 3)
+    m.check()
+
+
+def test_slots_lowest_first_zeroed_and_scratch():
+    m = manager([FULL], states=[StateNeed((2,), "float32")], storage=True, max_running=2)
+    s0, s1 = m.admit(10), m.admit(11)
+    assert (s0, s1) == (0, 1) and m.slots.scratch_slot == 2
+    state = m.slots.tensors[0]
+    assert state.shape == (3, 2)
+    state[0] = 7.0
+    assert not m.can_admit(None)
+    with pytest.raises(MemoryError):
+        m.admit(12)
+    m.release(10)
+    assert m.admit(13) == 0 and float(state[0].abs().sum()) == 0.0   # zeroed on assignment
+    m.check()
+
+
+def test_shared_prefix_pages():
+    m = manager([FULL], num_pages=6)
+    m.admit(1, total_tokens=5)
+    m.extend(1, 5)
+    first_two = m.table(0, 1)[:2]
+    m.admit(2, total_tokens=6, shared_pages=first_two)
+    assert m.lengths[2] == 4 and m.table(0, 2) == first_two
+    m.extend(2, 2)
+    assert m.table(0, 2)[:2] == first_two and m.table(0, 2)[2] not in m.table(0, 1)
+    m.release(1)
+    assert m.groups[0].allocator.ref_count(first_two[0]) == 1   # still held by request 2
+    m.release(2)
+    assert m.free_pages() == 6
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_orders_lose_no_page(seed):
+    """Requests arrive, grow by random portions, and end in random order; after every operation no page
+    is lost, held twice or freed twice, and at the end every page and slot is free."""
+    rng = random.Random(seed)
+    win = PagedKVNeed(2, 8, window=5)
+    m = manager([FULL, win], num_pages=40, page_size=4, max_running=4)
+    live, next_id = {}, 1
+    for _ in range(400):
+        action = rng.random()
+        if action < 0.25 and len(live) < 4:
+            total = rng.randint(1, 60)
+            reserve = rng.random() < 0.5
+            if m.can_admit(total if reserve else None, max_chunk=7):
+                m.admit(next_id, total if reserve else None, max_chunk=7)
+                live[next_id] = total
+                next_id += 1
+        elif action < 0.85 and live:
+            r = rng.choice(list(live))
+            room = live[r] - m.lengths[r]
+            if room > 0:
+                n = rng.randint(1, min(7, room))
+                try:
+                    m.extend(r, n)
+                except MemoryError:
+                    m.release(r)           # an unreserved request that found no page: give up cleanly
+                    del live[r]
+        elif live:
+            r = rng.choice(list(live))
+            m.release(r)
+            del live[r]
+        m.check()
+        for g in m.groups:
+            held = sum(len(g.allocator.pages_of(o)) for o in g.allocator.owners())
+            assert held + g.allocator.free_pages == g.num_pages
+    for r in list(live):
+        m.release(r)
+    m.check()
+    assert all(m.free_pages(g) == 40 for g in range(2)) and m.slots.free_slots == 4
+    assert all(g.allocator.reserved_pages == 0 for g in m.groups)

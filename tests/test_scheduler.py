@@ -1,0 +1,189 @@
+"""The scheduler's decisions and the engine around it, on the CPU with the torch twins of the kernels."""
+
+import pytest
+import torch
+
+import plain_llama as plain
+from helpers import TINIES, random_tokens, write_tiny_model
+from simple_inference_amd import Engine, EngineConfig, RequestState, SamplingParams
+from simple_inference_amd.engine import Request, Scheduler
+from simple_inference_amd.sampling import uniform_for
+from twins import TwinKernels
+
+
+def req(n_prompt, max_new=4):
+    return Request(prompt_tokens=list(range(1, n_prompt + 1)), params=SamplingParams(max_new_tokens=max_new))
+
+
+# ---- the scheduler alone ---------------------------------------------------------------------
+def test_admission_is_first_come_first_served_without_overtaking():
+    s = Scheduler(max_running=4, token_budget=1000, chunk_tokens=8)
+    a, b, c = req(5), req(50), req(2)
+    for r in (a, b, c):
+        s.add(r)
+    fits = lambda r: r.prompt_len < 10          # b cannot get its pages
+    assert s.admit(fits) == [a]
+    assert [r.state for r in (a, b, c)] == [RequestState.PREFILL, RequestState.WAITING, RequestState.WAITING]
+    assert s.admit(fits) == []                   # c does not jump over b
+    assert s.admit(lambda r: True) == [b, c]
+
+
+def test_token_budget_and_slots():
+    s = Scheduler(max_running=2, token_budget=10, chunk_tokens=8)
+    a, b, c = req(30), req(4), req(4)
+    for r in (a, b, c):
+        s.add(r)
+    assert s.admit() == [a]                      # an idle engine always admits one, however long
+    assert s.admit() == []                       # 30 + 4 > 10
+    a.state = RequestState.FINISHED
+    assert s.evict_finished() == [a]
+    assert s.admit() == [b, c] and s.admit() == []   # two slots
+
+
+def test_plan_gives_decoders_one_token_then_prompt_portions_in_order():
+    s = Scheduler(max_running=4, token_budget=1000, chunk_tokens=8)
+    d1, d2, p1, p2 = req(3), req(3), req(20), req(5)
+    for r in (d1, p1, d2, p2):
+        s.add(r)
+    s.admit()
+    d1.state = d2.state = RequestState.DECODE
+    p1.num_computed = 16
+    plan = s.plan_step()
+    assert [(r.id, n) for r, n in plan] == [(d1.id, 1), (d2.id, 1), (p1.id, 4), (p2.id, 2)]
+    p1.num_computed, p2.num_computed = 20, 2
+    p1.state = RequestState.DECODE
+    assert [(r.id, n) for r, n in s.plan_step()] == [(d1.id, 1), (p1.id, 1), (d2.id, 1), (p2.id, 3)]
+
+
+# ---- the engine on the CPU -----------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def folder(tmp_path_factory):
+    return write_tiny_model(tmp_path_factory.mktemp("sched"), TINIES["b"], seed=21)
+
+
+def engine(folder, **kw):
+    base = dict(device="cpu", dtype="float32", max_seq_len=128, block_size=8, max_running=4, chunk_tokens=16,
+                eos_id=-1)
+    base.update(kw)
+    return Engine.from_folder(folder, EngineConfig(**base), TwinKernels())
+
+
+def plain_greedy(folder, prompt, n):
+    cfg, w = plain.read_model(folder)
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(plain.forward(cfg, w, toks)[-1].argmax()))
+    return toks[len(prompt):]
+
+
+PROMPTS = [random_tokens(384, n, seed=40 + i) for i, n in enumerate((1, 17, 40, 70))]
+
+
+def test_tokens_do_not_depend_on_batching_queueing_or_portions(folder):
+    want = [plain_greedy(folder, p, 6) for p in PROMPTS]
+    for kw in (dict(max_running=1), dict(max_running=4), dict(max_running=2), dict(max_running=4, chunk_tokens=5),
+               dict(max_running=3, num_kv_blocks=24, chunk_tokens=64)):
+        eng = engine(folder, **kw)
+        reqs = [eng.add_request(p, max_new_tokens=6) for p in PROMPTS]
+        eng.run()
+        assert [r.generated for r in reqs] == want, kw
+        assert all(r.state is RequestState.FINISHED and r.slot is None for r in reqs)
+        assert eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks() and eng.cache.slots.free_slots == kw["max_running"]
+        eng.cache.check()
+
+
+def test_a_request_that_finds_no_pages_waits_for_a_finished_one(folder):
+    """serving/test_paged_kv_cache.py:247-269: 2 pages, two 3-token prompts with 1 new token each."""
+    eng = engine(folder, block_size=4, num_kv_blocks=1, max_running=2)
+    a = eng.add_request([1, 4, 6], max_new_tokens=1)
+    b = eng.add_request([1, 5, 9], max_new_tokens=1)
+    eng.step()
+    assert a.state is RequestState.FINISHED and b.state is RequestState.WAITING
+    eng.step()
+    assert b.state is RequestState.FINISHED and eng.cache.free_pages() == 1
+    assert a.generated == plain_greedy(folder, [1, 4, 6], 1) and b.generated == plain_greedy(folder, [1, 5, 9], 1)
+
+
+def test_first_token_comes_from_the_step_that_ends_the_prompt(folder):
+    eng = engine(folder, chunk_tokens=16)
+    r = eng.add_request(PROMPTS[2], max_new_tokens=3)       # 40 tokens: portions 16, 16, 8
+    emitted = [eng.step() for _ in range(3)]
+    assert emitted[0] == {} and emitted[1] == {} and list(emitted[2]) == [r.id]
+    assert r.state is RequestState.DECODE and r.num_computed == 40
+    eng.step()
+    assert r.num_generated == 2 and r.num_computed == 41
+
+
+def test_decoders_go_on_while_a_long_prompt_is_fed_in_portions(folder):
+    eng = engine(folder, chunk_tokens=9)
+    short = eng.add_request(PROMPTS[0], max_new_tokens=8)
+    eng.step()
+    long = eng.add_request(PROMPTS[3], max_new_tokens=2)     # 70 tokens at 8 a step beside the decoder
+    for _ in range(4):
+        out = eng.step()
+        assert short.id in out and long.id not in out
+    eng.run()
+    assert short.generated == plain_greedy(folder, PROMPTS[0], 8)
+    assert long.generated == plain_greedy(folder, PROMPTS[3], 2)
+
+
+def test_temperature_sampling_is_seeded_per_request_and_independent_of_the_batch(folder):
+    cfg, w = plain.read_model(folder)
+    params = [SamplingParams(temperature=0.8, seed=100 + i, max_new_tokens=6, top_k=k, top_p=p)
+              for i, (k, p) in enumerate(((0, 1.0), (5, 1.0), (0, 0.7), (20, 0.9)))]
+    want = []
+    for prompt, sp in zip(PROMPTS, params):
+        toks = list(prompt)
+        for n in range(6):
+            logits = plain.forward(cfg, w, toks)[-1]
+            toks.append(plain.sample_with_uniform(logits, uniform_for(sp.seed, n), sp.temperature, sp.top_k, sp.top_p))
+        want.append(toks[len(prompt):])
+    for kw in (dict(max_running=1), dict(max_running=4, chunk_tokens=7)):
+        eng = engine(folder, **kw)
+        reqs = [eng.add_request(p, params=sp) for p, sp in zip(PROMPTS, params)]
+        eng.run()
+        assert [r.generated for r in reqs] == want, kw
+    assert len({tuple(t) for t in want}) == 4
+
+
+def test_stops_at_eos_and_generate_does_not_yield_it(folder):
+    first = plain_greedy(folder, PROMPTS[1], 3)
+    eng = engine(folder, eos_id=first[2])
+    r = eng.add_request(PROMPTS[1], max_new_tokens=10)
+    eng.run()
+    assert r.generated == first and r.eos_hit                 # EOS is kept in generated (serving/engine.py:449-460)
+    eng = engine(folder, eos_id=first[2])
+    assert list(eng.generate(PROMPTS[1], max_new_tokens=10, temperature=0.0)) == first[:2]
+    ignoring = engine(folder, eos_id=first[2])
+    r = ignoring.add_request(PROMPTS[1], params=SamplingParams(max_new_tokens=5, ignore_eos=True))
+    ignoring.run()
+    assert r.num_generated == 5
+
+
+def test_add_request_checks(folder):
+    eng = engine(folder, max_seq_len=32, num_kv_blocks=2)
+    for prompt, new, word in (([], 1, "empty"), ([1, 2], 0, "max_new_tokens"), ([1] * 30, 3, "max_seq_len"),
+                              ([1] * 10, 10, "more pages"), ([1, 999], 2, "out-of-range")):
+        with pytest.raises(ValueError, match=word):
+            eng.add_request(prompt, max_new_tokens=new)
+
+
+def test_reset_gives_everything_back(folder):
+    eng = engine(folder)
+    for p in PROMPTS:
+        eng.add_request(p, max_new_tokens=4)
+    eng.step()
+    eng.reset()
+    assert not eng.has_work() and eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks()
+    r = eng.add_request(PROMPTS[1], max_new_tokens=2)
+    eng.run()
+    assert r.generated == plain_greedy(folder, PROMPTS[1], 2)
+
+
+def test_generate_with_stats_has_the_reference_names(folder):
+    eng = engine(folder)
+    tokens, stats = eng.generate_with_stats(PROMPTS[1], max_new_tokens=4, temperature=0.0)
+    assert tokens == plain_greedy(folder, PROMPTS[1], 4)
+    for key in ("ttft_ms", "tpot_ms", "prefill_ms", "decode_tok_s", "total_wall_ms", "total_tok_s", "peak_vram_gb",
+                "prompt_tokens", "new_tokens"):
+        assert key in stats
