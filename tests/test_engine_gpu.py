@@ -1,0 +1,108 @@
+"""The engine on the GPU: greedy generation through the entry points, graph replay, sampling."""
+
+import pytest
+import torch
+
+import plain_llama as plain
+from helpers import TINIES, random_tokens, rel_err, write_tiny_model
+from simple_inference_amd import Engine, EngineConfig, RequestState, SamplingParams
+from simple_inference_amd.engine import StepEntry
+from simple_inference_amd.sampling import uniform_for
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {n: write_tiny_model(tmp_path_factory.mktemp(f"eng_{n}"), t, seed=51) for n, t in TINIES.items()}
+
+
+def engine(folder, tiny, dtype, **kw):
+    base = dict(device="cuda:0", dtype=dtype, max_seq_len=256, block_size=tiny.page_size, max_running=4,
+                chunk_tokens=24, eos_id=-1)
+    base.update(kw)
+    return Engine.from_folder(folder, EngineConfig(**base))
+
+
+def greedy_matches_plain(folder, prompt, generated, dtype):
+    """Every generated token is the plain implementation's argmax, or (bfloat16) one whose logit ties with it."""
+    cfg, w = plain.read_model(folder)
+    toks = list(prompt)
+    for got in generated:
+        logits = plain.forward(cfg, w, toks)[-1]
+        want = int(logits.argmax())
+        if got != want:
+            margin = float(logits[want] - logits[got])
+            assert dtype == "bfloat16" and margin <= 2.5e-2 * float(logits.abs().max()), (got, want, margin)
+        toks.append(got)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(TINIES))
+def test_greedy_generation_through_the_entry_points(folders, name, dtype):
+    tiny = TINIES[name]
+    vocab = tiny.config["vocab_size"]
+    prompts = [random_tokens(vocab, n, seed=60 + i) for i, n in enumerate((1, 17, 40, 70))]
+    eng = engine(folders[name], tiny, dtype)
+    reqs = [eng.add_request(p, max_new_tokens=8) for p in prompts]
+    eng.run()
+    for p, r in zip(prompts, reqs):
+        assert r.state is RequestState.FINISHED and r.num_generated == 8
+        greedy_matches_plain(folders[name], p, r.generated, dtype)
+    assert eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks()
+    # the streaming entry point gives the same tokens as the batch did
+    solo = engine(folders[name], tiny, dtype, max_running=1)
+    assert list(solo.generate(prompts[2], max_new_tokens=8, temperature=0.0)) == reqs[2].generated
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_equals_eager_on_every_replay(folders, dtype):
+    """Replayed steps against the same steps run eagerly, with eager work and synchronisation between
+    replays, several batch buckets and a growing context."""
+    tiny = TINIES["b"]
+    vocab = tiny.config["vocab_size"]
+    prompts = [random_tokens(vocab, n, seed=70 + i) for i, n in enumerate((5, 33, 12))]
+    eager = engine(folders["b"], tiny, dtype, use_graphs=False)
+    graphed = engine(folders["b"], tiny, dtype, use_graphs=True)
+    ra = [eager.add_request(p, max_new_tokens=20 - 4 * i) for i, p in enumerate(prompts)]
+    rb = [graphed.add_request(p, max_new_tokens=20 - 4 * i) for i, p in enumerate(prompts)]
+    while eager.has_work() or graphed.has_work():
+        a, b = eager.step(), graphed.step()
+        torch.cuda.synchronize()
+        assert list(a.values()) == list(b.values())
+    assert [r.generated for r in ra] == [r.generated for r in rb]
+    assert graphed.graphs.replays >= 15 and len(graphed.graphs._made) >= 2       # buckets 4, 2, 1 as requests end
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_logits(folders, dtype):
+    tiny = TINIES["c"]
+    eng = engine(folders["c"], tiny, dtype, use_graphs=True)
+    prompt = random_tokens(tiny.config["vocab_size"], 50, seed=80)
+    eng.cache.admit(1)
+    eng.runner.run([StepEntry(1, prompt[:30], [])])
+    ref = plain.forward(*plain.read_model(folders["c"]), prompt)
+    for i in range(30, 50):
+        logits = eng.graphs.run([StepEntry(1, [prompt[i]], [0])])
+        assert rel_err(logits, ref[i:i + 1]) <= (2.5e-2 if dtype == "bfloat16" else 2e-5)
+
+
+def test_temperature_sampling_on_the_gpu_follows_the_request_seed(folders):
+    tiny = TINIES["a"]
+    cfg, w = plain.read_model(folders["a"])
+    prompts = [random_tokens(256, n, seed=90 + i) for i, n in enumerate((9, 13))]
+    params = [SamplingParams(temperature=0.8, seed=7 + i, max_new_tokens=6, top_k=k, top_p=p)
+              for i, (k, p) in enumerate(((0, 1.0), (12, 0.9)))]
+    outs = []
+    for kw in (dict(max_running=1), dict(max_running=2, chunk_tokens=4)):
+        eng = engine(folders["a"], tiny, "float32", **kw)
+        reqs = [eng.add_request(p, params=sp) for p, sp in zip(prompts, params)]
+        eng.run()
+        outs.append([r.generated for r in reqs])
+    assert outs[0] == outs[1]
+    for prompt, sp, got in zip(prompts, params, outs[0]):
+        toks = list(prompt)
+        for n, t in enumerate(got):
+            logits = plain.forward(cfg, w, toks)[-1]
+            assert t == plain.sample_with_uniform(logits, uniform_for(sp.seed, n), sp.temperature, sp.top_k, sp.top_p)
+            toks.append(t)

@@ -1,0 +1,229 @@
+"""Parts that are not the served architecture's, defined here and plugged in from outside.
+
+A toy mixer with state of its own, a layer order that names a layer twice, and a mixer that reads
+another layer's pages are registered, built and stepped without a change to the package's files.
+They run on the CPU with the torch twins and on the GPU with the HIP kernels.
+"""
+
+import copy
+
+import pytest
+import torch
+
+from helpers import rel_err
+from simple_inference_amd.cache import CacheManager
+from simple_inference_amd.config import EngineConfig, register_architecture, unregister_architecture
+from simple_inference_amd.engine import StepEntry, StepRunner, build_model
+from simple_inference_amd.parts import (
+    MIXERS, LayerSpec, ModelPlan, PartSpec, StateNeed, TensorSpec, register_mixer,
+)
+from simple_inference_amd.weights import random_tensors, target_dtype
+
+BACKENDS = [pytest.param("twins"), pytest.param("hip-f32", marks=pytest.mark.gpu),
+            pytest.param("hip-bf16", marks=pytest.mark.gpu)]
+
+
+class RunningMeanMixer:
+    """out[t] = W . mean(h[0..t]): the state is the running sum of the inputs, one row per request."""
+
+    def __init__(self, params, env):
+        self.hidden = int(params["hidden_size"])
+        self.env = env
+        self.w = None
+
+    def weight_specs(self):
+        return {"w": TensorSpec((self.hidden, self.hidden))}
+
+    def bind(self, tensors):
+        self.w = tensors["w"]
+
+    def cache_need(self):
+        return None
+
+    def state_need(self):
+        return StateNeed((self.hidden,), "float32")
+
+    def forward(self, h, ctx, cache):
+        means = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+        slots = ctx.state_slots.tolist()
+        positions = ctx.positions.tolist()
+        t = 0
+        for s, n in enumerate(ctx.q_lens):
+            running = cache.state[slots[s]]
+            for i in range(n):
+                running += h[t].float()
+                means[t] = running / (positions[t] + 1)
+                t += 1
+        return self.env.kernels.linear(means.to(h.dtype), self.w)
+
+
+H, V = 32, 64
+
+
+def toy_plan(cfg):
+    norm = lambda name: PartSpec("rmsnorm", {"size": H, "eps": 1e-5}, {"weight": name})
+    ffn = lambda p: PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 48},
+                             {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"})
+    rope = {"kind": "rope", "params": {"rotary_dim": 8, "theta": 10000.0, "scaling": None}}   # partial rotation
+    attn = lambda p, **extra: PartSpec(
+        "attention", dict({"hidden_size": H, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16, "position": rope}, **extra),
+        {k: f"{p}.{k}" for k in (("q", "o") if "kv_from_layer" in extra else ("q", "k", "v", "o"))})
+    layers = [
+        LayerSpec(mixer=attn("l0.attn", window=cfg.get("window")), feed_forward=ffn("l0.ffn"),
+                  mixer_norm=norm("l0.n1"), feed_forward_norm=norm("l0.n2")),
+        LayerSpec(mixer=PartSpec("test_running_mean", {"hidden_size": H}, {"w": "l1.mix.w"}), feed_forward=ffn("l1.ffn"),
+                  mixer_norm=norm("l1.n1"), feed_forward_norm=norm("l1.n2")),
+        LayerSpec(mixer=attn("l2.attn", kv_from_layer=0, window=cfg.get("window")), feed_forward=ffn("l2.ffn"),
+                  mixer_norm=norm("l2.n1"), feed_forward_norm=norm("l2.n2")),
+    ]
+    return ModelPlan(
+        hidden_size=H, vocab_size=V,
+        embedding=PartSpec("embedding", {"vocab_size": V, "hidden_size": H}, {"weight": "embed"}),
+        layers=layers, order=cfg.get("order", [0, 1, 2, 1]),   # layer 1 runs twice; each run has a state of its own
+        final_norm=norm("final"), head=PartSpec("head", {"vocab_size": V, "hidden_size": H, "tied": True}, {}),
+    )
+
+
+@pytest.fixture()
+def toy_registered():
+    register_mixer("test_running_mean", RunningMeanMixer, replace=True)
+    register_architecture("ToyForTests", lambda d: d, toy_plan, replace=True)
+    yield
+    unregister_architecture("ToyForTests")
+    MIXERS.unregister("test_running_mean")
+
+
+def make(backend, cfg, page_size=4, num_pages=32):
+    if backend == "twins":
+        from twins import TwinKernels
+        kernels, device, dtype = TwinKernels(), "cpu", "float32"
+    else:
+        from simple_inference_amd.kernels import HipKernels
+        kernels, device = HipKernels(), "cuda:0"
+        dtype = "float32" if backend == "hip-f32" else "bfloat16"
+    ecfg = EngineConfig(device=device, dtype=dtype, max_seq_len=128, block_size=page_size, max_running=3)
+    model, _ = build_model(cfg, ecfg, kernels)
+    expected = model.expected_tensors()
+    drawn = random_tensors(expected, seed=3, std=0.15, gain_std=0.1)
+    model.bind({k: t.to(device=device, dtype=target_dtype(t.dtype, expected[k].role, ecfg.torch_dtype))
+                for k, t in drawn.items()})
+    cache = CacheManager(model.cache_layout(), page_size=page_size, num_pages=num_pages, max_running=3,
+                         dtype=ecfg.torch_dtype, device=device)
+    return StepRunner(model, cache, kernels, device, 128), cache, drawn
+
+
+def toy_reference(w, tokens, order, window):
+    """The toy model, whole sequence, in float64, written out plainly."""
+    import plain_llama as plain
+    w = {k: v.double() for k, v in w.items()}
+    T = len(tokens)
+    x = w["embed"][tokens]
+    pos = torch.arange(T)
+    inv = plain.rope_inv_freq(8, 10000.0)
+    cos, sin = plain.rope_tables(pos, inv, torch.float64)
+
+    def rot(t):  # the first 8 of 16 dims rotate
+        return torch.cat([plain.apply_rope(t[..., :8], cos, sin), t[..., 8:]], dim=-1)
+
+    kv0 = None
+    for li in order:
+        p = f"l{li}"
+        h = plain.rms_norm(x, w[f"{p}.n1"], 1e-5)
+        if li == 1:
+            mean = h.cumsum(0) / (pos[:, None] + 1)
+            a = mean @ w["l1.mix.w"].T
+        else:
+            q = rot((h @ w[f"{p}.attn.q"].T).view(T, 4, 16))
+            if li == 0:
+                kv0 = (rot((h @ w["l0.attn.k"].T).view(T, 2, 16)), (h @ w["l0.attn.v"].T).view(T, 2, 16))
+            a = plain.attention(q, kv0[0], kv0[1], pos, pos, window=window).reshape(T, 64) @ w[f"{p}.attn.o"].T
+        x = x + a
+        h = plain.rms_norm(x, w[f"{p}.n2"], 1e-5)
+        x = x + plain.swiglu_mlp(h, w[f"{p}.ffn.gate"], w[f"{p}.ffn.up"], w[f"{p}.ffn.down"])
+    return plain.rms_norm(x, w["final"], 1e-5) @ w["embed"].T
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("window", [None, 6])
+def test_toy_architecture_is_registered_built_and_stepped(toy_registered, backend, window):
+    cfg = {"architectures": ["ToyForTests"], "window": window}
+    runner, cache, weights = make(backend, cfg)
+    layout = runner.model.cache_layout()
+    assert len(layout.states) == 2 and layout.run_state == [None, 0, None, 1]      # a state per run of layer 1
+    assert layout.run_kv[0] == layout.run_kv[2] and layout.run_kv[1] is None          # layer 2 reads layer 0's pages
+    assert layout.kv_slabs == [1]
+
+    g = torch.Generator().manual_seed(0)
+    seqs = {r: torch.randint(0, V, (n,), generator=g).tolist() for r, n in ((1, 23), (2, 9), (3, 15))}
+    want = {r: toy_reference(weights, t, [0, 1, 2, 1], window) for r, t in seqs.items()}
+    tol = 3e-2 if backend == "hip-bf16" else 2e-5
+
+    # whole, alone
+    for r, toks in seqs.items():
+        cache.admit(r)
+        out = runner.run([StepEntry(r, toks, list(range(len(toks))))])
+        assert rel_err(out, want[r]) <= tol
+        cache.release(r)
+    # in portions, mixed with each other, slots and pages handed out again
+    cuts = {1: [5, 1, 9, 2, 6], 2: [2, 7], 3: [1, 1, 13]}
+    fed = {r: 0 for r in seqs}
+    got = {r: [] for r in seqs}
+    for r in seqs:
+        cache.admit(r)
+    while any(cuts.values()):
+        entries = []
+        for r in seqs:
+            if cuts[r]:
+                n = cuts[r].pop(0)
+                entries.append(StepEntry(r, seqs[r][fed[r]:fed[r] + n], list(range(n))))
+                fed[r] += n
+        out = runner.run(entries)
+        i = 0
+        for e in entries:
+            got[e.req].append(out[i:i + len(e.tokens)])
+            i += len(e.tokens)
+    for r in seqs:
+        assert rel_err(torch.cat(got[r]), want[r]) <= tol
+        cache.release(r)
+    cache.check()
+    assert cache.free_pages() == 32 and cache.slots.free_slots == 3
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_each_run_of_a_layer_has_pages_of_its_own(toy_registered, backend):
+    """Order [0, 0, 1]: the attention layer runs twice; its second run must not see the keys of the first."""
+    def plan(cfg):
+        p = toy_plan(cfg)
+        p.layers = p.layers[:2]
+        p.order = [0, 0, 1]
+        return p
+    register_architecture("ToyTwice", lambda d: d, plan, replace=True)
+    try:
+        runner, cache, weights = make(backend, {"architectures": ["ToyTwice"]})
+        assert runner.model.cache_layout().kv_slabs == [2]
+        toks = torch.randint(0, V, (19,), generator=torch.Generator().manual_seed(1)).tolist()
+
+        import plain_llama as plain
+        w = {k: v.double() for k, v in weights.items()}
+        T, pos = len(toks), torch.arange(len(toks))
+        inv = plain.rope_inv_freq(8, 10000.0)
+        cos, sin = plain.rope_tables(pos, inv, torch.float64)
+        rot = lambda t: torch.cat([plain.apply_rope(t[..., :8], cos, sin), t[..., 8:]], dim=-1)
+        x = w["embed"][toks]
+        for li in (0, 0):
+            h = plain.rms_norm(x, w["l0.n1"], 1e-5)
+            q, k = rot((h @ w["l0.attn.q"].T).view(T, 4, 16)), rot((h @ w["l0.attn.k"].T).view(T, 2, 16))
+            v = (h @ w["l0.attn.v"].T).view(T, 2, 16)
+            x = x + plain.attention(q, k, v, pos, pos).reshape(T, 64) @ w["l0.attn.o"].T
+            x = x + plain.swiglu_mlp(plain.rms_norm(x, w["l0.n2"], 1e-5), w["l0.ffn.gate"], w["l0.ffn.up"], w["l0.ffn.down"])
+        h = plain.rms_norm(x, w["l1.n1"], 1e-5)
+        x = x + (h.cumsum(0) / (pos[:, None] + 1)) @ w["l1.mix.w"].T
+        x = x + plain.swiglu_mlp(plain.rms_norm(x, w["l1.n2"], 1e-5), w["l1.ffn.gate"], w["l1.ffn.up"], w["l1.ffn.down"])
+        want = plain.rms_norm(x, w["final"], 1e-5) @ w["embed"].T
+
+        cache.admit(1)
+        got = torch.cat([runner.run([StepEntry(1, toks[a:b], list(range(b - a)))])
+                         for a, b in ((0, 7), (7, 8), (8, 19))])
+        assert rel_err(got, want) <= (3e-2 if backend == "hip-bf16" else 2e-5)
+    finally:
+        unregister_architecture("ToyTwice")
