@@ -1,0 +1,89 @@
+"""Prefix reuse: the reference's vectors for its radix cache, and the engine with it (CPU, twins)."""
+
+import pytest
+import torch
+
+from helpers import TINIES, random_tokens, write_tiny_model
+from simple_inference_amd import Engine, EngineConfig
+from simple_inference_amd.cache import CacheManager, PrefixCache
+from simple_inference_amd.parts.model import CacheLayout
+from simple_inference_amd.parts.plan import PagedKVNeed
+from twins import TwinKernels
+
+
+def manager(num_pages, page_size=2, window=None):
+    lay = CacheLayout()
+    lay.kv_groups, lay.kv_slabs, lay.run_kv, lay.run_state = [PagedKVNeed(1, 4, window)], [1], [(0, 0)], [None]
+    return CacheManager(lay, page_size=page_size, num_pages=num_pages, max_running=4, dtype=torch.float32,
+                        device="cpu", allocate_storage=False)
+
+
+def test_match_shares_complete_pages_and_clear_keeps_live_requests():
+    """serving/test_paged_kv_cache.py:93-125: free pages 4 -> 4 -> 6."""
+    m = manager(6)
+    pc = PrefixCache(m, max_pages=6)
+    m.admit(1, total_tokens=4)
+    m.extend(1, 4)
+    pc.insert([1, 2, 3, 4], m.table(0, 1))
+    assert m.free_pages() == 4
+    pages = pc.match([1, 2, 3, 4, 5])
+    assert pages == m.table(0, 1) and pc.stats()["matched_tokens"] == 4
+    assert pc.match([1, 2, 3, 4]) == m.table(0, 1)[:1]          # a token must be left to run
+    assert pc.match([9, 9, 9]) == []
+    m.admit(2, total_tokens=6, shared_pages=pages)
+    assert m.lengths[2] == 4 and m.free_pages() == 4
+    m.release(1)
+    assert m.free_pages() == 4                                   # still pinned by the cache and request 2
+    pc.clear()
+    assert m.free_pages() == 4                                   # request 2 still holds them
+    m.release(2)
+    assert m.free_pages() == 6
+    m.check()
+
+
+def test_least_recently_used_leaf_goes_first():
+    """serving/test_paged_kv_cache.py:127-156: max 2 pages; the newer path evicts the old one."""
+    m = manager(8)
+    pc = PrefixCache(m, max_pages=2)
+    for rid, toks in ((1, [1, 2, 3, 4]), (2, [5, 6, 7, 8])):
+        m.admit(rid, total_tokens=4)
+        m.extend(rid, 4)
+        pc.insert(toks, m.table(0, rid))
+        m.release(rid)
+    assert pc.match([1, 2, 3, 4, 0]) == [] and len(pc.match([5, 6, 7, 8, 0])) == 2
+    assert pc.stats()["evictions"] == 2 and pc.stats()["cached_blocks"] == 2
+    assert m.free_pages() == 6
+    assert pc.evict_until_available(8) and m.free_pages() == 8
+    assert not pc.evict_until_available(9)
+
+
+def test_refuses_models_it_cannot_serve():
+    with pytest.raises(ValueError, match="window"):
+        PrefixCache(manager(4, window=8), max_pages=4)
+
+
+def test_engine_with_prefix_reuse_gives_the_same_tokens(tmp_path):
+    """serving/test_paged_kv_cache.py:271-301 in kind: the second prompt shares pages with the first."""
+    tiny = TINIES["b"]
+    folder = write_tiny_model(tmp_path, tiny, seed=61)
+    base = random_tokens(384, 37, seed=1)
+    prompts = [base + [5, 6], base + [7], base[:20] + [9, 9, 9], random_tokens(384, 11, seed=2)]
+
+    def run(use):
+        eng = Engine.from_folder(folder, EngineConfig(
+            device="cpu", dtype="float32", max_seq_len=96, block_size=8, max_running=2, chunk_tokens=16, eos_id=-1,
+            num_kv_blocks=24, use_prefix_cache=use, prefix_cache_blocks=6), TwinKernels())
+        out = []
+        for p in prompts:                       # one after the other, so that earlier prompts are cached
+            r = eng.add_request(p, max_new_tokens=4)
+            eng.run()
+            out.append((r.generated, r.cached_prefix_len))
+        return eng, out
+    _, plain_out = run(False)
+    eng, cached_out = run(True)
+    assert [g for g, _ in cached_out] == [g for g, _ in plain_out]
+    assert [c for _, c in cached_out] == [0, 32, 16, 0]        # whole pages of 8, one token always left to run
+    assert eng.prefix_cache.stats()["hits"] == 2 and eng.prefix_cache.stats()["cached_blocks"] <= 6
+    eng.cache.check()
+    eng.reset()
+    assert eng.cache.free_pages() == 24
