@@ -171,3 +171,16 @@ def test_long_decoding(folders, backend):
     schedule = [([(0, tokens[:4], [3])], [])] + [([(0, [t], [0])], []) for t in tokens[4:]]
     got = replay(runner, cache, schedule)
     check_against_plain(got, {0: tokens}, folders["a"], backend)
+
+
+@pytest.mark.gpu
+def test_float32_stored_weights_in_the_bfloat16_engine(tmp_path):
+    """A tensor stored in 32 bit stays so: its products run in float32 between bfloat16 activations."""
+    tiny = TINIES["a"]
+    folder = write_tiny_model(tmp_path, tiny, seed=4, storage="float32")
+    runner, cache, mcfg = make_runner(folder, "hip-bf16", tiny.page_size, num_pages=64)
+    assert runner.model.embedding.weight.dtype == torch.float32
+    assert runner.model.layers[0].mixer.w_qkv.dtype == torch.float32
+    tokens = random_tokens(mcfg.vocab_size, 40, seed=3)
+    got = replay(runner, cache, [([(0, tokens[:33], list(range(33)))], []), ([(0, tokens[33:], list(range(7)))], [0])])
+    check_against_plain(got, {0: tokens}, folder, "hip-bf16")
