@@ -223,25 +223,39 @@ def test_matrix_core_attention_decode_and_mixed(hip, geom):
         torch.testing.assert_close(plain_kernel.float(), ref.float(), **tol(dtype))
 
 
-def test_attention_finds_a_far_key(hip):
-    """One key among hundreds is made to stand out; the output must be its value row."""
-    n_heads, n_kv, D, ps = 2, 1, 64, 16
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("q_len", [1, 40])
+def test_attention_finds_one_key_at_every_kind_of_edge(hip, dtype, q_len):
+    """One key among hundreds is made to stand out; the output must be its value row.  The key is put at
+    the edges where an indexing fault would lose it: first and last offset of a page, of a 32- and
+    64-key tile, of a 256-key split, the first key, the newest key, and both sides of a window's edge."""
+    n_heads, n_kv, D, ps = 4, 2, 64, 16
     kv = 700
-    ctx = Ctx([1], [kv])
-    cache = Cache(64, n_kv, ps, D, torch.float32, [kv])
-    cache.k_pages.copy_(0.01 * rnd(*cache.k_pages.shape, seed=1))
-    cache.v_pages.copy_(rnd(*cache.v_pages.shape, seed=2))
-    far = 37
-    page = int(cache.block_table[0, far // ps])
+    ctx = Ctx([q_len], [kv])
+    last = kv - 1                       # the position of the last query
     direction = torch.nn.functional.normalize(rnd(D, seed=3), dim=0)
-    cache.k_pages[page, 0, far % ps] = 40.0 * direction
-    qkv = torch.zeros(1, (n_heads + 2 * n_kv) * D, device=DEV)
-    qkv[0, :D] = 40.0 * direction
-    qkv[0, D:2 * D] = 40.0 * direction
-    out = hip.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), None, ctx, cache)
-    want = cache.v_pages[page, 0, :, far % ps]
-    torch.testing.assert_close(out[0, :D], want, rtol=1e-4, atol=1e-4)
-    torch.testing.assert_close(out[0, D:], want, rtol=1e-4, atol=1e-4)
+    base_k = 0.01 * rnd(64, n_kv, ps, D, seed=1)
+    values = rnd(64, n_kv, D, ps, seed=2)
+    qkv = torch.zeros(q_len, (n_heads + 2 * n_kv) * D)
+    qkv[:, :n_heads * D] = (30.0 * direction).repeat(n_heads)
+    qkv = qkv.to(dtype).to(DEV)
+    cache = Cache(64, n_kv, ps, D, dtype, [kv])
+    cache.v_pages.copy_(values.to(dtype))
+    window = 300
+    edge = last - window + 1            # oldest key the last query sees through the window
+    for far, win, seen in [(0, None, True), (15, None, True), (16, None, True), (31, None, True), (32, None, True),
+                           (63, None, True), (64, None, True), (255, None, True), (256, None, True),
+                           (511, None, True), (512, None, True), (last - q_len, None, True), (last, None, True),
+                           (edge, window, True), (edge - 1, window, False), (edge + 1, window, True)]:
+        cache.k_pages.copy_(base_k.to(dtype))
+        page = int(cache.block_table[0, far // ps])
+        cache.k_pages[page, :, far % ps] = (30.0 * direction).to(dtype)
+        out = hip.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), win, ctx, cache).float()
+        row = out[-1].view(n_heads, D)      # the last query sees every key up to ``last``
+        for h in range(n_heads):
+            want = cache.v_pages[page, h // 2, :, far % ps].float()
+            close = torch.allclose(row[h], want, rtol=2e-2, atol=2e-2)
+            assert close == seen, (far, win, h)
 
 
 @pytest.mark.parametrize("vocab", [16, 1000, 128256])
