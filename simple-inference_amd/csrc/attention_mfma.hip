@@ -30,7 +30,8 @@
 //          split; the query heads that share the kv head are the q columns (at most 16).  The four
 //          partial results are merged through LDS; (m, l, acc) per split go to a workspace and a
 //          second kernel combines the splits in order.
-// prefill: one wave per 16*NQ consecutive tokens of one query head; 4 waves a workgroup.
+// prefill: one wave per 16*NQ consecutive tokens of one query head; 4 waves a workgroup, which share
+//          each tile of keys and values through LDS (two stages; head sizes whose stages fit 64 KiB).
 #include "common.h"
 
 #ifndef SIA_HEAD_DIM
@@ -52,9 +53,16 @@ __device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
 __device__ __forceinline__ bf16x8 zero8() {
     return __builtin_bit_cast(bf16x8, make_uint4(0u, 0u, 0u, 0u));
 }
+// Two floats to two bfloat16 (round to nearest even) with the hardware's packed conversion.
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2;
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+    const floatx2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
+// 2^x by the hardware instruction; arguments here are <= 0 or -inf, results in [0, 1].
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+constexpr float LOG2E = 1.4426950408889634f;
 
 // 64 consecutive entries of a sequence's block table, one per lane.
 struct PageWindow {
@@ -109,13 +117,67 @@ __device__ __forceinline__ void load_stage(Stage& st, const bf16_t* __restrict__
     for (int db = 0; db < DBLOCKS; ++db) st.v[db] = load8(vbase + (size_t)(db * 16 + r) * ps);
 }
 
-// Scores, online softmax and value product of one loaded tile, for NQ groups of 16 q columns.
+// Masks the scores of a tile, updates the running softmax statistics of each q column, rescales the
+// accumulators and returns the tile's probabilities as the P^T operand.
 //   lo[n], hi[n]: visible keys of this lane's column in group n (hi < lo: none).
+//   scale_log2 = scale * log2(e) > 0: exponentials are taken as 2^(s * scale_log2 - m), and the running
+//   maximum m is kept in those units, so a score costs one fused multiply-add and one exp2.
+// A tile that every column of the wave sees whole skips the masking, and the accumulators are rescaled
+// only when some column's maximum moved (both tests are wave-uniform).
+template <int NQ>
+__device__ __forceinline__ void softmax_update(floatx4 (&s)[NQ][2], int kb, const int (&lo)[NQ], const int (&hi)[NQ],
+                                               float scale_log2, float (&m)[NQ], float (&l)[NQ],
+                                               floatx4 (&acc)[NQ][DBLOCKS], bf16x8 (&p)[NQ]) {
+    const int g = (threadIdx.x & 63) >> 4;
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+        if (!__all(kb >= lo[n] && kb + TILE - 1 <= hi[n])) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = kb + g * 8 + h * 4 + i;
+                    if (key < lo[n] || key > hi[n]) s[n][h][i] = -INFINITY;
+                }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(s[n][0][0], s[n][0][1]), fmaxf(s[n][0][2], s[n][0][3])),
+                         fmaxf(fmaxf(s[n][1][0], s[n][1][1]), fmaxf(s[n][1][2], s[n][1][3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, SIA_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, SIA_WAVE));
+        const float m_new = fmaxf(m[n], mx * scale_log2);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
+        const float alpha = fast_exp2(m[n] - m_use);
+        float sum = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float e = fast_exp2(fmaf(s[n][h][i], scale_log2, -m_use));
+                s[n][h][i] = e;
+                sum += e;
+            }
+        sum += __shfl_xor(sum, 16, SIA_WAVE);
+        sum += __shfl_xor(sum, 32, SIA_WAVE);
+        l[n] = l[n] * alpha + sum;
+        m[n] = m_new;
+        if (__any(alpha != 1.f)) {
+#pragma unroll
+            for (int db = 0; db < DBLOCKS; ++db) acc[n][db] *= alpha;
+        }
+        uint4 u;
+        u.x = pack2(s[n][0][0], s[n][0][1]);
+        u.y = pack2(s[n][0][2], s[n][0][3]);
+        u.z = pack2(s[n][1][0], s[n][1][1]);
+        u.w = pack2(s[n][1][2], s[n][1][3]);
+        p[n] = __builtin_bit_cast(bf16x8, u);
+    }
+}
+
+// Scores, online softmax and value product of one tile held in registers.
 template <int NQ>
 __device__ __forceinline__ void compute_stage(const Stage& st, const bf16x8 (&q)[NQ][KSTEPS], int kb,
                                               const int (&lo)[NQ], const int (&hi)[NQ], float scale,
                                               float (&m)[NQ], float (&l)[NQ], floatx4 (&acc)[NQ][DBLOCKS]) {
-    const int g = (threadIdx.x & 63) >> 4;
     floatx4 s[NQ][2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -128,45 +190,7 @@ __device__ __forceinline__ void compute_stage(const Stage& st, const bf16x8 (&q)
                 s[n][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.k[h][ks], q[n][ks], s[n][h], 0, 0, 0);
     }
     bf16x8 p[NQ];
-#pragma unroll
-    for (int n = 0; n < NQ; ++n) {
-        float mx = -INFINITY;
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = kb + g * 8 + h * 4 + i;
-                const float v = (key >= lo[n] && key <= hi[n]) ? s[n][h][i] * scale : -INFINITY;
-                s[n][h][i] = v;
-                mx = fmaxf(mx, v);
-            }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, SIA_WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, SIA_WAVE));
-        const float m_new = fmaxf(m[n], mx);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
-        const float alpha = __expf(m[n] - m_use);
-        float sum = 0.f;
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float e = __expf(s[n][h][i] - m_use);
-                s[n][h][i] = e;
-                sum += e;
-            }
-        sum += __shfl_xor(sum, 16, SIA_WAVE);
-        sum += __shfl_xor(sum, 32, SIA_WAVE);
-        l[n] = l[n] * alpha + sum;
-        m[n] = m_new;
-#pragma unroll
-        for (int db = 0; db < DBLOCKS; ++db) acc[n][db] *= alpha;
-        uint4 u;
-        u.x = pack2(s[n][0][0], s[n][0][1]);
-        u.y = pack2(s[n][0][2], s[n][0][3]);
-        u.z = pack2(s[n][1][0], s[n][1][1]);
-        u.w = pack2(s[n][1][2], s[n][1][3]);
-        p[n] = __builtin_bit_cast(bf16x8, u);
-    }
+    softmax_update<NQ>(s, kb, lo, hi, scale, m, l, acc, p);
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db)
 #pragma unroll
@@ -175,6 +199,8 @@ __device__ __forceinline__ void compute_stage(const Stage& st, const bf16x8 (&q)
 }
 
 // All tiles that meet [range_lo, range_hi] (range_lo <= range_hi), two register stages in turn.
+// The block-table window (64 entries) is loaded outside the pipelined loop, once per 64 pages: a load
+// inside it would make every iteration wait for all outstanding loads.
 template <int NQ>
 __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], const bf16_t* __restrict__ kp,
                                              const bf16_t* __restrict__ vp, const int* __restrict__ table,
@@ -183,26 +209,21 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], cons
                                              float (&m)[NQ], float (&l)[NQ], floatx4 (&acc)[NQ][DBLOCKS]) {
     const int lane = threadIdx.x & 63;
     const int kb_first = (range_lo / TILE) * TILE, kb_last = (range_hi / TILE) * TILE;
-    PageWindow pages;
-    pages_load(pages, table, table_width, range_lo >> ps_log2, lane);
-    // Before a tile is loaded the window must hold its entries; it is moved when a tile's last entry
-    // lies beyond it (every 64 pages).
-    auto ensure = [&](int kb) {
-        const int last_entry = min(kb + TILE - 1, range_hi) >> ps_log2;
-        if (last_entry >= pages.base + SIA_WAVE)
-            pages_load(pages, table, table_width, max(kb, range_lo) >> ps_log2, lane);
-    };
-    Stage a, b;
-    load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, kb_first, range_lo, range_hi);
-    for (int kb = kb_first; kb <= kb_last; kb += 2 * TILE) {
-        const int kb1 = min(kb + TILE, kb_last);  // past the end: the last tile again, never computed
-        ensure(kb1);
-        load_stage(b, kp, vp, pages, ps_log2, n_kv, hk, kb1, range_lo, range_hi);
-        compute_stage<NQ>(a, q, kb, lo, hi, scale, m, l, acc);
-        const int kb2 = min(kb + 2 * TILE, kb_last);
-        ensure(kb2);
-        load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, kb2, range_lo, range_hi);
-        if (kb + TILE <= kb_last) compute_stage<NQ>(b, q, kb + TILE, lo, hi, scale, m, l, acc);
+    const int window_keys = SIA_WAVE << ps_log2;  // a multiple of TILE: tiles do not straddle windows
+    for (int w_first = kb_first; w_first <= kb_last; w_first += window_keys) {
+        const int w_last = min(kb_last, w_first + window_keys - TILE);
+        PageWindow pages;
+        pages_load(pages, table, table_width, w_first >> ps_log2, lane);
+        Stage a, b;
+        load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, w_first, range_lo, range_hi);
+        for (int kb = w_first; kb <= w_last; kb += 2 * TILE) {
+            const int kb1 = min(kb + TILE, w_last);  // past the end: the last tile again, never computed
+            load_stage(b, kp, vp, pages, ps_log2, n_kv, hk, kb1, range_lo, range_hi);
+            compute_stage<NQ>(a, q, kb, lo, hi, scale, m, l, acc);
+            const int kb2 = min(kb + 2 * TILE, w_last);
+            load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, kb2, range_lo, range_hi);
+            if (kb + TILE <= w_last) compute_stage<NQ>(b, q, kb + TILE, lo, hi, scale, m, l, acc);
+        }
     }
 }
 
@@ -228,6 +249,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     extern __shared__ float lds[];  // [DEC_WAVES][group][HD + 2]
     const int split = blockIdx.x, hk = blockIdx.y, seq = blockIdx.z;
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    scale *= LOG2E;  // exponentials are taken as powers of two
     const int pos = kv_len[seq] - 1;
     const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
     const int s_lo = max(lo_all, split * split_keys);
@@ -275,7 +297,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
 #pragma unroll
         for (int w = 0; w < DEC_WAVES; ++w) {
             const float* row = lds + (size_t)(w * group + c) * ROW;
-            const float wgt = __expf(row[HD] - mx);  // a wave without keys has m = -inf: weight 0
+            const float wgt = fast_exp2(row[HD] - mx);  // a wave without keys has m = -inf: weight 0
             o += wgt * row[d];
             lsum += wgt * row[HD + 1];
         }
@@ -289,7 +311,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
 }
 
 // Combines the splits of each (sequence, head): out = sum_s w_s acc_s / sum_s w_s l_s with
-// w_s = exp(m_s - max m), summed in split order, eight splits' loads in flight at a time.
+// w_s = 2^(m_s - max m) (the maxima are kept in units of log2), summed in split order, eight splits' loads in flight at a time.
 __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
     const float* __restrict__ ws_acc, const float* __restrict__ ws_ml, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int window, int split_keys,
@@ -316,7 +338,7 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
         for (int j = 0; j < 8; ++j) {
             const int s = min(s0 + j, last);  // a clamped slot is read again with weight 0
             const bool live = s0 + j <= last;
-            w[j] = live ? __expf(ws_ml[(base + s) * 2] - mx) : 0.f;
+            w[j] = live ? fast_exp2(ws_ml[(base + s) * 2] - mx) : 0.f;
             denom += live ? w[j] * ws_ml[(base + s) * 2 + 1] : 0.f;
 #pragma unroll
             for (int dd = 0; dd < DD; ++dd) {
@@ -342,30 +364,142 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
 // ---------------------------------------------------------------------------------------------------
 // prefill: runs of several tokens (works for single tokens too, without splitting the keys)
 // ---------------------------------------------------------------------------------------------------
-constexpr int PF_NQ = 2;                        // groups of 16 tokens per wave
+constexpr int PF_NQ = HD <= 128 ? 2 : 1;        // groups of 16 tokens per wave
 constexpr int PF_WAVES = 4;
 constexpr int PF_ROWS = PF_WAVES * PF_NQ * 16;  // tokens per workgroup
+constexpr int PF_THREADS = PF_WAVES * SIA_WAVE;
+// Key and value tiles are shared by the workgroup's waves through LDS (two stages).  Rows are padded by
+// 16 bytes so that the 16 lanes of a 128-bit read hit 64 different banks.
+constexpr int K_STRIDE = HD + 8;                // elements per key row
+constexpr int V_STRIDE = TILE + 8;              // elements per dim row (32 positions + pad)
+constexpr int K_CHUNKS = TILE * HD / 8;         // 16-byte pieces of a key tile
+constexpr int PF_PER_THREAD = (K_CHUNKS + PF_THREADS - 1) / PF_THREADS;
+constexpr bool PF_USE_LDS = (2 * (TILE * K_STRIDE + HD * V_STRIDE) * 2) <= 64 * 1024;
 
-__global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
+// What one thread carries from global memory to LDS for one tile.
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;  // a plain 16-byte register value
+struct TileRegs {
+    u32x4 k[PF_PER_THREAD];
+    u32x4 v[PF_PER_THREAD];
+};
+
+// Issues the global loads of the tile at kb.  Key chunk c is (key c / (HD/8), dims 8 (c % (HD/8)) ..);
+// value chunks are ordered (page segment, dim, group of 8 positions), so that consecutive threads read
+// consecutive 16 bytes of a page.  Keys outside [lo, hi] are clamped into it (see load_stage).
+__device__ __forceinline__ void tile_fetch(TileRegs& t, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
+                                           const PageWindow& pages, int ps_log2, int n_kv, int hk, int kb, int lo,
+                                           int hi) {
+    const int ps = 1 << ps_log2;
+    const int t_lo = max(kb, lo), t_hi = min(kb + TILE - 1, hi);
+    const int seg_keys = min(ps, TILE);            // positions of one page inside a tile
+    const int seg_chunks = HD * (seg_keys / 8);    // 16-byte pieces of one page's values inside a tile
+#pragma unroll
+    for (int i = 0; i < PF_PER_THREAD; ++i) {
+        const int c = threadIdx.x + i * PF_THREADS;
+        if (K_CHUNKS % PF_THREADS != 0 && c >= K_CHUNKS) break;
+        {
+            const int key = min(max(kb + c / (HD / 8), t_lo), t_hi);
+            const int page = pages_get(pages, key >> ps_log2);
+            t.k[i] = *reinterpret_cast<const u32x4*>(kp + (((size_t)page * n_kv + hk) * ps + (key & (ps - 1))) * HD +
+                                                     (c % (HD / 8)) * 8);
+        }
+        {
+            const int seg = c / seg_chunks, rest = c % seg_chunks;
+            const int d = rest / (seg_keys / 8), j = rest % (seg_keys / 8);
+            const int key0 = min(max(kb + seg * seg_keys + j * 8, t_lo & ~7), t_hi & ~7);
+            const int page = pages_get(pages, key0 >> ps_log2);
+            t.v[i] = *reinterpret_cast<const u32x4*>(vp + (((size_t)page * n_kv + hk) * HD + d) * ps + (key0 & (ps - 1)));
+        }
+    }
+}
+
+// Writes a fetched tile into an LDS stage.  Key rows are stored in the order the score MFMAs read them
+// (row 16h + m holds key 8(m/4) + 4h + m%4), so that the 16 lanes of a read take 16 consecutive rows.
+__device__ __forceinline__ void tile_store(const TileRegs& t, bf16_t* __restrict__ k_lds, bf16_t* __restrict__ v_lds,
+                                           int ps_log2) {
+    const int ps = 1 << ps_log2;
+    const int seg_keys = min(ps, TILE);
+    const int seg_chunks = HD * (seg_keys / 8);
+#pragma unroll
+    for (int i = 0; i < PF_PER_THREAD; ++i) {
+        const int c = threadIdx.x + i * PF_THREADS;
+        if (K_CHUNKS % PF_THREADS != 0 && c >= K_CHUNKS) break;
+        const int key = c / (HD / 8);
+        const int row = ((key >> 2) & 1) * 16 + (key >> 3) * 4 + (key & 3);
+        *reinterpret_cast<u32x4*>(k_lds + row * K_STRIDE + (c % (HD / 8)) * 8) = t.k[i];
+        const int seg = c / seg_chunks, rest = c % seg_chunks;
+        const int d = rest / (seg_keys / 8), j = rest % (seg_keys / 8);
+        *reinterpret_cast<u32x4*>(v_lds + d * V_STRIDE + seg * seg_keys + j * 8) = t.v[i];
+    }
+}
+
+// Scores, online softmax and value product of one tile held in an LDS stage; every operand is read
+// right before the MFMAs that use it.
+template <int NQ>
+__device__ __forceinline__ void compute_from_lds(const bf16_t* __restrict__ k_lds, const bf16_t* __restrict__ v_lds,
+                                                 const bf16x8 (&q)[NQ][KSTEPS], int kb, const int (&lo)[NQ],
+                                                 const int (&hi)[NQ], float scale, float (&m)[NQ], float (&l)[NQ],
+                                                 floatx4 (&acc)[NQ][DBLOCKS]) {
+    const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    floatx4 s[NQ][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int n = 0; n < NQ; ++n) s[n][h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            const int d0 = ks * 32 + g * 8;
+            bf16x8 a;
+            if (HD % 32 == 0 || ks < KSTEPS - 1)
+                a = load8(k_lds + (h * 16 + r) * K_STRIDE + d0);
+            else
+                a = d0 < HD ? load8(k_lds + (h * 16 + r) * K_STRIDE + d0) : zero8();
+#pragma unroll
+            for (int n = 0; n < NQ; ++n) s[n][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[n][ks], s[n][h], 0, 0, 0);
+        }
+    }
+    bf16x8 p[NQ];
+    softmax_update<NQ>(s, kb, lo, hi, scale, m, l, acc, p);
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) {
+        const bf16x8 a = load8(v_lds + (db * 16 + r) * V_STRIDE + g * 8);
+#pragma unroll
+        for (int n = 0; n < NQ; ++n) acc[n][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p[n], acc[n][db], 0, 0, 0);
+    }
+}
+
+__global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale,
     int window, int seq_begin, int seq_end) {
-    // which sequence and which of its row tiles this workgroup has
-    int tile = blockIdx.x, seq = seq_begin;
+    // The chip has 8 dies (XCDs), each with an L2 of its own, and hands workgroups to them in turn.  The
+    // workgroup ids are renumbered so that each die gets a contiguous range: the query heads that share a
+    // kv head, and the row tiles of one head, then read their keys and values through one L2.
+    scale *= LOG2E;  // exponentials are taken as powers of two
+    const int n_blocks = gridDim.x * gridDim.y;
+    int vid = blockIdx.y * gridDim.x + blockIdx.x;
+    if (n_blocks % 8 == 0) vid = (vid % 8) * (n_blocks / 8) + vid / 8;
+    const int head = vid / gridDim.x;
+    // which sequence and which of its row tiles this workgroup has; late tiles (most keys) come first
+    int tile = vid % gridDim.x, seq = seq_begin;
     for (; seq < seq_end; ++seq) {
         const int tiles = (cu_q[seq + 1] - cu_q[seq] + PF_ROWS - 1) / PF_ROWS;
-        if (tile < tiles) break;
+        if (tile < tiles) {
+            tile = tiles - 1 - tile;
+            break;
+        }
         tile -= tiles;
     }
     if (seq >= seq_end) return;
-    const int head = blockIdx.y, hk = head / (n_heads / n_kv);
+    const int hk = head / (n_heads / n_kv);
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int q_begin = cu_q[seq], q_len = cu_q[seq + 1] - q_begin;
     const int first_pos = kv_len[seq] - q_len;
     const int row0 = tile * PF_ROWS + wave * PF_NQ * 16;  // this wave's first row within the sequence's run
-    if (row0 >= q_len) return;
+    const bool wave_live = row0 < q_len;
     const int row_last = min(q_len - 1, row0 + PF_NQ * 16 - 1);
+    const int* table = block_table + (size_t)seq * table_width;
 
     bf16x8 qf[PF_NQ][KSTEPS];
     int lo[PF_NQ], hi[PF_NQ];
@@ -384,10 +518,56 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
 #pragma unroll
         for (int db = 0; db < DBLOCKS; ++db) acc[n][db] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    const int range_hi = first_pos + row_last;
-    const int range_lo = window > 0 ? max(0, first_pos + row0 - window + 1) : 0;
-    attend_range<PF_NQ>(qf, kp, vp, block_table + (size_t)seq * table_width, table_width, ps_log2, n_kv, hk,
-                        range_lo, range_hi, lo, hi, scale, m, l, acc);
+
+    if constexpr (PF_USE_LDS) {
+        __shared__ __align__(16) bf16_t k_lds[2][TILE * K_STRIDE];
+        __shared__ __align__(16) bf16_t v_lds[2][HD * V_STRIDE];
+        // the workgroup's key range: from the first row's oldest visible key to the last live row's position
+        const int blk_rows = min(q_len - tile * PF_ROWS, PF_ROWS);
+        const int blk_hi = first_pos + tile * PF_ROWS + blk_rows - 1;
+        const int blk_lo = window > 0 ? max(0, first_pos + tile * PF_ROWS - window + 1) : 0;
+        const int wave_hi = first_pos + row_last;
+        const int wave_lo = window > 0 ? max(0, first_pos + row0 - window + 1) : 0;
+        const int kb_first = (blk_lo / TILE) * TILE, kb_last = (blk_hi / TILE) * TILE;
+        // Two register sets: while tile t is computed from LDS, tile t+1 waits in one set (its loads were
+        // issued an iteration ago) and the loads of tile t+2 are issued into the other.  The block-table
+        // window is loaded outside the pipelined loop, once per 64 pages.
+        const int window_keys = SIA_WAVE << ps_log2;
+        for (int w_first = kb_first; w_first <= kb_last; w_first += window_keys) {
+            const int w_last = min(kb_last, w_first + window_keys - TILE);
+            PageWindow pages;
+            pages_load(pages, table, table_width, w_first >> ps_log2, lane);
+            TileRegs regs_a, regs_b;
+// One tile step: issue the loads of tile kb + 2 tiles into FREE, compute tile kb from LDS stage STAGE,
+// write the tile that waits in NEXT into the other stage.  (A macro, not a lambda: register sets that a
+// closure captures by reference end up in scratch memory.)
+#define PF_STEP(FREE, NEXT, KB, STAGE)                                                                          \
+    do {                                                                                                        \
+        tile_fetch(FREE, kp, vp, pages, ps_log2, n_kv, hk, min((KB) + 2 * TILE, w_last), blk_lo, blk_hi);       \
+        if (wave_live && (KB) <= wave_hi && (KB) + TILE - 1 >= wave_lo)                                         \
+            compute_from_lds<PF_NQ>(k_lds[STAGE], v_lds[STAGE], qf, (KB), lo, hi, scale, m, l, acc);            \
+        if ((KB) + TILE <= w_last) tile_store(NEXT, k_lds[(STAGE) ^ 1], v_lds[(STAGE) ^ 1], ps_log2);           \
+        __syncthreads();                                                                                        \
+    } while (0)
+            tile_fetch(regs_a, kp, vp, pages, ps_log2, n_kv, hk, w_first, blk_lo, blk_hi);
+            tile_fetch(regs_b, kp, vp, pages, ps_log2, n_kv, hk, min(w_first + TILE, w_last), blk_lo, blk_hi);
+            tile_store(regs_a, k_lds[0], v_lds[0], ps_log2);
+            __syncthreads();
+            for (int kb = w_first; kb <= w_last; kb += 2 * TILE) {
+                PF_STEP(regs_a, regs_b, kb, 0);
+                if (kb + TILE <= w_last) PF_STEP(regs_b, regs_a, kb + TILE, 1);
+            }
+#undef PF_STEP
+        }
+    } else {
+        if (wave_live) {
+            const int range_hi = first_pos + row_last;
+            const int range_lo = window > 0 ? max(0, first_pos + row0 - window + 1) : 0;
+            attend_range<PF_NQ>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, range_lo, range_hi, lo, hi, scale,
+                                m, l, acc);
+        }
+    }
+    if (!wave_live) return;
 
 #pragma unroll
     for (int n = 0; n < PF_NQ; ++n) {

@@ -269,7 +269,7 @@ class HipKernels:
         out = torch.empty((n, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
         page = cache.page_size
         if (self.use_mfma_attention and qkv.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256
-                and page >= 8 and width % 8 == 0):
+                and page >= 8 and width % 8 == 0 and scale > 0):
             self._mfma_attention(qkv, out, n_heads, n_kv_heads, head_dim, scale, int(window or 0), ctx, cache)
             return out
         self._check(self.core.sia_attention_generic(

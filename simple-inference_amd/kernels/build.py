@@ -31,6 +31,9 @@ HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # MFMA results in ordinary vector registers: the attention kernels rescale and exponentiate them, and
+    # with accumulation registers every such touch costs two extra moves.
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
 
 # name -> sources.  "core" is everything a model needs in either dtype; further libraries
