@@ -32,6 +32,39 @@ template <typename T> __device__ __forceinline__ T from_float(float x);
 template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float x) { return float_to_bf16(x); }
 
+// Eight consecutive elements of a row as one register value: 32 bytes of float or 16 of bfloat16.
+template <typename T> struct Vec8;
+template <> struct Vec8<float> {
+    float4 a, b;
+    __device__ __forceinline__ void load(const float* p) { a = *(const float4*)p; b = *(const float4*)(p + 4); }
+    __device__ __forceinline__ void store(float* p) const { *(float4*)p = a; *(float4*)(p + 4) = b; }
+    __device__ __forceinline__ void get(float (&x)[8]) const {
+        x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+    }
+    __device__ __forceinline__ void set(const float (&x)[8]) {
+        a = make_float4(x[0], x[1], x[2], x[3]); b = make_float4(x[4], x[5], x[6], x[7]);
+    }
+};
+template <> struct Vec8<bf16_t> {
+    uint4 u;
+    __device__ __forceinline__ void load(const bf16_t* p) { u = *(const uint4*)p; }
+    __device__ __forceinline__ void store(bf16_t* p) const { *(uint4*)p = u; }
+    __device__ __forceinline__ void get(float (&x)[8]) const {
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            x[2 * i] = __uint_as_float(w[i] << 16);
+            x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+    __device__ __forceinline__ void set(const float (&x)[8]) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = (uint32_t)float_to_bf16(x[2 * i]) | ((uint32_t)float_to_bf16(x[2 * i + 1]) << 16);
+        u = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+};
+
 // Butterfly reductions over the 64 lanes of a wave: every lane gets the result, and the
 // order of additions is fixed, so a row's result does not depend on what else is in a batch.
 __device__ __forceinline__ float wave_sum(float v) {

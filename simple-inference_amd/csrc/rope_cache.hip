@@ -61,6 +61,73 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
     }
 }
 
+// The same with 8 elements a thread (head_dim, rotary_dim / 2 and the row stride multiples of 8): a work
+// item is a pair of 8-element pieces (i, i + rotary_dim / 2) of a q or k head, an unrotated piece of a k
+// head, or a piece of a v head.  All of a token's loads are independent of one another.
+template <typename T>
+__global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ cos_table,
+                                         const float* __restrict__ sin_table, const int* __restrict__ positions,
+                                         const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
+                                         int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                         int n_heads, int n_kv, int head_dim, int rotary_dim, int page_size) {
+    const int n = blockIdx.x;
+    const int pos = positions[n];
+    const int half = rotary_dim / 2, pairs = half / 8, plain = (head_dim - rotary_dim) / 8, pieces = head_dim / 8;
+    T* row = qkv + (size_t)n * row_stride;
+    const float* cs = cos_table + (size_t)pos * half;
+    const float* sn = sin_table + (size_t)pos * half;
+    int page = -1, off = 0;
+    if (n_kv > 0) {
+        page = block_table[(size_t)seq_of_token[n] * table_width + pos / page_size];
+        off = pos % page_size;
+    }
+    const int items_q = n_heads * pairs, items_kr = n_kv * pairs, items_kp = n_kv * plain, items_v = n_kv * pieces;
+    for (int item = threadIdx.x; item < items_q + items_kr + items_kp + items_v; item += blockDim.x) {
+        if (item < items_q + items_kr) {  // a rotated pair of q (in place) or of k (into the page)
+            const bool is_q = item < items_q;
+            const int it = is_q ? item : item - items_q;
+            const int h = it / pairs, j = (it % pairs) * 8;
+            T* x = row + (is_q ? h : n_heads + h) * head_dim;
+            Vec8<T> va, vb;
+            Vec8<float> vc, vs;
+            va.load(x + j);
+            vb.load(x + j + half);
+            vc.load(cs + j);
+            vs.load(sn + j);
+            float a[8], b[8], c[8], s[8], ra[8], rb[8];
+            va.get(a); vb.get(b); vc.get(c); vs.get(s);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                ra[i] = a[i] * c[i] - b[i] * s[i];
+                rb[i] = b[i] * c[i] + a[i] * s[i];
+            }
+            va.set(ra);
+            vb.set(rb);
+            if (is_q) {
+                va.store(x + j);
+                vb.store(x + j + half);
+            } else if (page >= 0) {
+                T* dst = k_pages + (((size_t)page * n_kv + h) * page_size + off) * head_dim;
+                va.store(dst + j);
+                vb.store(dst + j + half);
+            }
+        } else if (item < items_q + items_kr + items_kp) {  // dims of k beyond the rotation
+            const int it = item - items_q - items_kr;
+            const int h = it / plain, j = rotary_dim + (it % plain) * 8;
+            Vec8<T> v;
+            v.load(row + (n_heads + h) * head_dim + j);
+            if (page >= 0) v.store(k_pages + (((size_t)page * n_kv + h) * page_size + off) * head_dim + j);
+        } else if (page >= 0) {  // v: 8 dims, each to its own row of the page (positions are innermost there)
+            const int it = item - items_q - items_kr - items_kp;
+            const int h = it / pieces, j = (it % pieces) * 8;
+            const T* x = row + (n_heads + n_kv + h) * head_dim + j;
+            T* dst = v_pages + (((size_t)page * n_kv + h) * head_dim + j) * page_size + off;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dst[(size_t)i * page_size] = x[i];
+        }
+    }
+}
+
 SIA_EXPORT int sia_rope_kv_write(void* qkv, int row_stride, const float* cos_table, const float* sin_table,
                                  const int* positions, const int* seq_of_token, const int* block_table,
                                  int table_width, void* k_pages, void* v_pages, int n_tokens, int n_heads,
@@ -70,11 +137,21 @@ SIA_EXPORT int sia_rope_kv_write(void* qkv, int row_stride, const float* cos_tab
     if (rotary_dim < 0 || rotary_dim > head_dim || (rotary_dim & 1)) return SIA_BAD_ARGUMENT;
     if (n_kv > 0 && (!k_pages || !v_pages || !block_table || page_size <= 0)) return SIA_BAD_ARGUMENT;
     if (rotary_dim > 0 && (!cos_table || !sin_table)) return SIA_BAD_ARGUMENT;
-    dim3 grid(n_tokens), block(256);
-#define LAUNCH(T)                                                                                         \
-    hipLaunchKernelGGL(rope_kv_write_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride, cos_table,   \
-                       sin_table, positions, seq_of_token, block_table, table_width, (T*)k_pages,         \
-                       (T*)v_pages, n_heads, n_kv, head_dim, rotary_dim, page_size)
+    dim3 grid(n_tokens);
+    const bool vec = head_dim % 8 == 0 && rotary_dim % 16 == 0 && row_stride % 8 == 0;
+    const int items = vec ? (n_heads + n_kv) * (rotary_dim / 16) + n_kv * ((head_dim - rotary_dim) / 8 + head_dim / 8) : 0;
+    dim3 block(vec ? min(1024, max(SIA_WAVE, (items + SIA_WAVE - 1) / SIA_WAVE * SIA_WAVE)) : 256);
+#define LAUNCH(T)                                                                                             \
+    do {                                                                                                      \
+        if (vec)                                                                                              \
+            hipLaunchKernelGGL(rope_kv_write_vec_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride,      \
+                               cos_table, sin_table, positions, seq_of_token, block_table, table_width,       \
+                               (T*)k_pages, (T*)v_pages, n_heads, n_kv, head_dim, rotary_dim, page_size);     \
+        else                                                                                                  \
+            hipLaunchKernelGGL(rope_kv_write_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride,          \
+                               cos_table, sin_table, positions, seq_of_token, block_table, table_width,       \
+                               (T*)k_pages, (T*)v_pages, n_heads, n_kv, head_dim, rotary_dim, page_size);     \
+    } while (0)
     if (dtype == SIA_F32) LAUNCH(float);
     else if (dtype == SIA_BF16) LAUNCH(bf16_t);
     else return SIA_BAD_ARGUMENT;
