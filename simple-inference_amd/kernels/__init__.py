@@ -36,6 +36,7 @@ _SIGNATURES = {
     "sia_sample": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "sia_gemm_skinny": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_gemm_skinny_max_rows": [],
+    "sia_gemm_skinny_swiglu": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
 }
 
 
@@ -181,6 +182,20 @@ class HipKernels:
         if back is not None and not out_float32:
             y = self.cast(y, back)
         return y
+
+    def gated_linear(self, x, w_gate_up):
+        """``silu(x Wg^T) * (x Wu^T)`` for ``w_gate_up = [Wg; Wu]``: one kernel for few rows, else product + SwiGLU."""
+        self._want(x, "gated linear input")
+        self._want(w_gate_up, "gate/up weight")
+        M, K = x.shape
+        two_i = w_gate_up.shape[0]
+        if (self.use_skinny_gemm and x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
+                and M <= self._skinny_rows and two_i % 32 == 0 and K % 64 == 0 and w_gate_up.shape[1] == K):
+            y = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=x.device)
+            self._check(self.core.sia_gemm_skinny_swiglu(_ptr(x), _ptr(w_gate_up), _ptr(y), M, two_i // 2, K,
+                                                         self._stream()), "gemm_skinny_swiglu")
+            return y
+        return self.swiglu(self.linear(x, w_gate_up))
 
     def gemm_generic(self, x, w, out_float32=False):
         """The plain kernel for either dtype (tests compare it with the library product)."""

@@ -38,6 +38,5 @@ class SwiGLU:
 
     def forward(self, h, ctx):
         k = self.env.kernels
-        gu = k.linear(h, self.w_gate_up)
-        a = k.swiglu(gu)
+        a = k.gated_linear(h, self.w_gate_up)   # the activation is fused into the product where a kernel has it
         return k.linear(a, self.w_down)

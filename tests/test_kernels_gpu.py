@@ -144,6 +144,19 @@ def test_gemm_skinny(hip, shape):
     assert torch.equal(hip.linear(x[:1].contiguous(), w), out16[:1])
 
 
+@pytest.mark.parametrize("shape", [(1, 32, 64), (8, 8192, 3072), (16, 1008, 512), (5, 96, 320), (40, 128, 256)])
+def test_gated_linear(hip, shape):
+    """The product with the SwiGLU activation in its epilogue (few rows) or after it, against the twin."""
+    M, inter, K = shape
+    x = rnd(M, K, dtype=torch.bfloat16, seed=1)
+    w = rnd(2 * inter, K, dtype=torch.bfloat16, seed=2, scale=1 / math.sqrt(K))
+    gu = x.double() @ w.double().T
+    ref = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    out = hip.gated_linear(x, w)
+    assert out.shape == (M, inter) and out.dtype == torch.bfloat16
+    torch.testing.assert_close(out.double(), ref, rtol=2e-2, atol=2e-2)
+
+
 def test_float32_product_has_no_reduced_precision(hip):
     """An operand bit below bfloat16 (8 bits) and tf32 (10 bits) resolution must reach the product."""
     K = 8

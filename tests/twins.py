@@ -40,6 +40,9 @@ class TwinKernels:
         y = x.float() @ w.float().T
         return y if out_float32 else y.to(x.dtype)
 
+    def gated_linear(self, x, w_gate_up):
+        return self.swiglu(self.linear(x, w_gate_up))
+
     # -- feed-forward activation --------------------------------------------
     def swiglu(self, gu):
         inter = gu.shape[-1] // 2
