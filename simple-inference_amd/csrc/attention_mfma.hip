@@ -198,9 +198,30 @@ __device__ __forceinline__ void compute_stage(const Stage& st, const bf16x8 (&q)
             acc[n][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.v[db], p[n], acc[n][db], 0, 0, 0);
 }
 
-// All tiles that meet [range_lo, range_hi] (range_lo <= range_hi), two register stages in turn.
-// The block-table window (64 entries) is loaded outside the pipelined loop, once per 64 pages: a load
-// inside it would make every iteration wait for all outstanding loads.
+// The tiles w_first, w_first + TILE, ..., w_last, whose block-table entries the window holds; two register
+// stages in turn: the loads of tile t+1 are issued before the arithmetic of tile t.
+template <int NQ>
+__device__ __forceinline__ void attend_tiles(const PageWindow& pages, int w_first, int w_last,
+                                             const bf16x8 (&q)[NQ][KSTEPS], const bf16_t* __restrict__ kp,
+                                             const bf16_t* __restrict__ vp, int ps_log2, int n_kv, int hk,
+                                             int range_lo, int range_hi, const int (&lo)[NQ], const int (&hi)[NQ],
+                                             float scale, float (&m)[NQ], float (&l)[NQ],
+                                             floatx4 (&acc)[NQ][DBLOCKS]) {
+    Stage a, b;
+    load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, w_first, range_lo, range_hi);
+    for (int kb = w_first; kb <= w_last; kb += 2 * TILE) {
+        const int kb1 = min(kb + TILE, w_last);  // past the end: the last tile again, never computed
+        load_stage(b, kp, vp, pages, ps_log2, n_kv, hk, kb1, range_lo, range_hi);
+        compute_stage<NQ>(a, q, kb, lo, hi, scale, m, l, acc);
+        const int kb2 = min(kb + 2 * TILE, w_last);
+        load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, kb2, range_lo, range_hi);
+        if (kb + TILE <= w_last) compute_stage<NQ>(b, q, kb + TILE, lo, hi, scale, m, l, acc);
+    }
+}
+
+// All tiles that meet [range_lo, range_hi] (range_lo <= range_hi).  The block-table window (64 entries) is
+// loaded outside the pipelined loop, once per 64 pages: a load inside it would make every iteration wait
+// for all outstanding loads.
 template <int NQ>
 __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], const bf16_t* __restrict__ kp,
                                              const bf16_t* __restrict__ vp, const int* __restrict__ table,
@@ -211,19 +232,10 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], cons
     const int kb_first = (range_lo / TILE) * TILE, kb_last = (range_hi / TILE) * TILE;
     const int window_keys = SIA_WAVE << ps_log2;  // a multiple of TILE: tiles do not straddle windows
     for (int w_first = kb_first; w_first <= kb_last; w_first += window_keys) {
-        const int w_last = min(kb_last, w_first + window_keys - TILE);
         PageWindow pages;
         pages_load(pages, table, table_width, w_first >> ps_log2, lane);
-        Stage a, b;
-        load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, w_first, range_lo, range_hi);
-        for (int kb = w_first; kb <= w_last; kb += 2 * TILE) {
-            const int kb1 = min(kb + TILE, w_last);  // past the end: the last tile again, never computed
-            load_stage(b, kp, vp, pages, ps_log2, n_kv, hk, kb1, range_lo, range_hi);
-            compute_stage<NQ>(a, q, kb, lo, hi, scale, m, l, acc);
-            const int kb2 = min(kb + 2 * TILE, w_last);
-            load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, kb2, range_lo, range_hi);
-            if (kb + TILE <= w_last) compute_stage<NQ>(b, q, kb + TILE, lo, hi, scale, m, l, acc);
-        }
+        attend_tiles<NQ>(pages, w_first, min(kb_last, w_first + window_keys - TILE), q, kp, vp, ps_log2, n_kv, hk,
+                         range_lo, range_hi, lo, hi, scale, m, l, acc);
     }
 }
 
@@ -250,16 +262,25 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const int split = blockIdx.x, hk = blockIdx.y, seq = blockIdx.z;
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     scale *= LOG2E;  // exponentials are taken as powers of two
+    const int group = n_heads / n_kv;
+    const int part = split_keys / DEC_WAVES;
+    const int nominal = split * split_keys + wave * part;  // first key of this wave's quarter
+    const int* table = block_table + (size_t)seq * table_width;
+    // What does not depend on the sequence's length is loaded at once, beside the length itself: the
+    // block-table entries of the quarter, and the queries (sequence s's one token is row s of the batch).
+    const bool one_window = (part >> ps_log2) <= SIA_WAVE;
+    PageWindow pages;
+    pages_load(pages, table, table_width, nominal >> ps_log2, lane);
+    bf16x8 qf[1][KSTEPS];
+    load_q(qf[0], r < group ? q + (size_t)seq * q_row_stride + (hk * group + r) * HD : nullptr, g);
+
     const int pos = kv_len[seq] - 1;
     const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
     const int s_lo = max(lo_all, split * split_keys);
     const int s_hi = min(pos, split * split_keys + split_keys - 1);
     if (s_hi < s_lo) return;  // the whole workgroup: this split holds no visible key
-
-    const int group = n_heads / n_kv;
-    const int part = split_keys / DEC_WAVES;
-    const int w_lo = max(s_lo, split * split_keys + wave * part);
-    const int w_hi = min(s_hi, split * split_keys + wave * part + part - 1);
+    const int w_lo = max(s_lo, nominal);
+    const int w_hi = min(s_hi, nominal + part - 1);
 
     float m[1] = {-INFINITY}, l[1] = {0.f};
     floatx4 acc[1][DBLOCKS];
@@ -267,12 +288,12 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     for (int db = 0; db < DBLOCKS; ++db) acc[0][db] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     if (w_lo <= w_hi) {  // wave-uniform
-        const int token = cu_q[seq];
-        bf16x8 qf[1][KSTEPS];
-        load_q(qf[0], r < group ? q + (size_t)token * q_row_stride + (hk * group + r) * HD : nullptr, g);
         const int lo[1] = {r < group ? w_lo : 1}, hi[1] = {r < group ? w_hi : 0};
-        attend_range<1>(qf, kp, vp, block_table + (size_t)seq * table_width, table_width, ps_log2, n_kv, hk, w_lo,
-                        w_hi, lo, hi, scale, m, l, acc);
+        if (one_window)
+            attend_tiles<1>(pages, (w_lo / TILE) * TILE, (w_hi / TILE) * TILE, qf, kp, vp, ps_log2, n_kv, hk, w_lo,
+                            w_hi, lo, hi, scale, m, l, acc);
+        else
+            attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, m, l, acc);
     }
 
     constexpr int ROW = HD + 2;
@@ -596,7 +617,8 @@ static int log2_exact(int v) {
 
 SIA_EXPORT int sia_attn_mfma_head_dim() { return HD; }
 
-// Sequences 0 .. n_seqs-1 of the step, each with exactly one new token.  ws_acc holds
+// Sequences 0 .. n_seqs-1 of the step, each with exactly one new token, which is row s of q (cu_q[s] = s).
+// ws_acc holds
 // n_seqs * n_heads * max_splits * head_dim floats and ws_ml twice n_seqs * n_heads * max_splits;
 // max_splits * split_keys must cover the longest sequence; split_keys is a multiple of 128.
 SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
