@@ -219,9 +219,9 @@ __device__ __forceinline__ void attend_tiles(const PageWindow& pages, int w_firs
     }
 }
 
-// All tiles that meet [range_lo, range_hi] (range_lo <= range_hi).  The block-table window (64 entries) is
-// loaded outside the pipelined loop, once per 64 pages: a load inside it would make every iteration wait
-// for all outstanding loads.
+// All tiles that meet [range_lo, range_hi] (range_lo <= range_hi).  The block-table window (64 entries,
+// starting at the page of the first tile it serves) is loaded outside the pipelined loop, once per 64
+// pages: a load inside it would make every iteration wait for all outstanding loads.
 template <int NQ>
 __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], const bf16_t* __restrict__ kp,
                                              const bf16_t* __restrict__ vp, const int* __restrict__ table,
@@ -230,12 +230,14 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], cons
                                              float (&m)[NQ], float (&l)[NQ], floatx4 (&acc)[NQ][DBLOCKS]) {
     const int lane = threadIdx.x & 63;
     const int kb_first = (range_lo / TILE) * TILE, kb_last = (range_hi / TILE) * TILE;
-    const int window_keys = SIA_WAVE << ps_log2;  // a multiple of TILE: tiles do not straddle windows
-    for (int w_first = kb_first; w_first <= kb_last; w_first += window_keys) {
+    for (int w_first = kb_first; w_first <= kb_last;) {
+        const int first_page = w_first >> ps_log2;
+        const int w_end = (first_page + SIA_WAVE) << ps_log2;  // first key beyond the window, a multiple of TILE
         PageWindow pages;
-        pages_load(pages, table, table_width, w_first >> ps_log2, lane);
-        attend_tiles<NQ>(pages, w_first, min(kb_last, w_first + window_keys - TILE), q, kp, vp, ps_log2, n_kv, hk,
-                         range_lo, range_hi, lo, hi, scale, m, l, acc);
+        pages_load(pages, table, table_width, first_page, lane);
+        attend_tiles<NQ>(pages, w_first, min(kb_last, w_end - TILE), q, kp, vp, ps_log2, n_kv, hk, range_lo, range_hi,
+                         lo, hi, scale, m, l, acc);
+        w_first = w_end;
     }
 }
 
@@ -257,43 +259,36 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, float* __restrict__ ws_acc, float* __restrict__ ws_ml, int n_heads, int n_kv,
-    int ps_log2, float scale, int window, int split_keys, int max_splits) {
+    int ps_log2, float scale, int window) {
     extern __shared__ float lds[];  // [DEC_WAVES][group][HD + 2]
-    const int split = blockIdx.x, hk = blockIdx.y, seq = blockIdx.z;
+    const int split = blockIdx.x, n_splits = gridDim.x, hk = blockIdx.y, seq = blockIdx.z;
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     scale *= LOG2E;  // exponentials are taken as powers of two
     const int group = n_heads / n_kv;
-    const int part = split_keys / DEC_WAVES;
-    const int nominal = split * split_keys + wave * part;  // first key of this wave's quarter
     const int* table = block_table + (size_t)seq * table_width;
-    // What does not depend on the sequence's length is loaded at once, beside the length itself: the
-    // block-table entries of the quarter, and the queries (sequence s's one token is row s of the batch).
-    const bool one_window = (part >> ps_log2) <= SIA_WAVE;
-    PageWindow pages;
-    pages_load(pages, table, table_width, nominal >> ps_log2, lane);
+    // The queries do not depend on the sequence's length: they are loaded beside it (sequence s's one token
+    // is row s of the batch).
     bf16x8 qf[1][KSTEPS];
     load_q(qf[0], r < group ? q + (size_t)seq * q_row_stride + (hk * group + r) * HD : nullptr, g);
 
+    // The tiles that hold visible keys are dealt evenly, in order, to the n_splits * DEC_WAVES waves that
+    // work for this (sequence, kv head): every wave gets a contiguous run, runs differ by one tile at most.
     const int pos = kv_len[seq] - 1;
     const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
-    const int s_lo = max(lo_all, split * split_keys);
-    const int s_hi = min(pos, split * split_keys + split_keys - 1);
-    if (s_hi < s_lo) return;  // the whole workgroup: this split holds no visible key
-    const int w_lo = max(s_lo, nominal);
-    const int w_hi = min(s_hi, nominal + part - 1);
+    const int t_first = lo_all / TILE, n_tiles = pos / TILE - t_first + 1;
+    const int n_waves = n_splits * DEC_WAVES, wi = split * DEC_WAVES + wave;
+    const int my_first = t_first + (int)(((long long)wi * n_tiles) / n_waves);
+    const int my_end = t_first + (int)(((long long)(wi + 1) * n_tiles) / n_waves);
 
     float m[1] = {-INFINITY}, l[1] = {0.f};
     floatx4 acc[1][DBLOCKS];
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) acc[0][db] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    if (w_lo <= w_hi) {  // wave-uniform
+    if (my_first < my_end) {  // wave-uniform
+        const int w_lo = max(lo_all, my_first * TILE), w_hi = min(pos, my_end * TILE - 1);
         const int lo[1] = {r < group ? w_lo : 1}, hi[1] = {r < group ? w_hi : 0};
-        if (one_window)
-            attend_tiles<1>(pages, (w_lo / TILE) * TILE, (w_hi / TILE) * TILE, qf, kp, vp, ps_log2, n_kv, hk, w_lo,
-                            w_hi, lo, hi, scale, m, l, acc);
-        else
-            attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, m, l, acc);
+        attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, m, l, acc);
     }
 
     constexpr int ROW = HD + 2;
@@ -314,15 +309,16 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
         float mx = -INFINITY;
 #pragma unroll
         for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, lds[(size_t)(w * group + c) * ROW + HD]);
+        const float mx_use = (mx == -INFINITY) ? 0.f : mx;  // no wave had a key: all weights 0, the split counts for nothing
         float o = 0.f, lsum = 0.f;
 #pragma unroll
         for (int w = 0; w < DEC_WAVES; ++w) {
             const float* row = lds + (size_t)(w * group + c) * ROW;
-            const float wgt = fast_exp2(row[HD] - mx);  // a wave without keys has m = -inf: weight 0
+            const float wgt = fast_exp2(row[HD] - mx_use);  // a wave without keys has m = -inf: weight 0
             o += wgt * row[d];
             lsum += wgt * row[HD + 1];
         }
-        const size_t slot = ((size_t)seq * n_heads + hk * group + c) * max_splits + split;
+        const size_t slot = ((size_t)seq * n_heads + hk * group + c) * n_splits + split;
         ws_acc[slot * HD + d] = o;
         if (d == 0) {
             ws_ml[slot * 2] = mx;
@@ -332,16 +328,14 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
 }
 
 // Combines the splits of each (sequence, head): out = sum_s w_s acc_s / sum_s w_s l_s with
-// w_s = 2^(m_s - max m) (the maxima are kept in units of log2), summed in split order, eight splits' loads in flight at a time.
+// w_s = 2^(m_s - max m) (the maxima are kept in units of log2; a split without keys has m = -inf and weight
+// 0), summed in split order, eight splits' loads in flight at a time.
 __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
     const float* __restrict__ ws_acc, const float* __restrict__ ws_ml, const int* __restrict__ cu_q,
-    const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int window, int split_keys,
-    int max_splits) {
+    bf16_t* __restrict__ out, int n_heads, int n_splits) {
     const int head = blockIdx.x, seq = blockIdx.y, lane = threadIdx.x;
-    const int pos = kv_len[seq] - 1;
-    const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
-    const int first = lo_all / split_keys, last = pos / split_keys;
-    const size_t base = ((size_t)seq * n_heads + head) * max_splits;
+    const int first = 0, last = n_splits - 1;
+    const size_t base = ((size_t)seq * n_heads + head) * n_splits;
     float mx = -INFINITY;
     for (int s0 = first; s0 <= last; s0 += SIA_WAVE) {
         const int s = s0 + lane;
@@ -552,12 +546,13 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
         const int kb_first = (blk_lo / TILE) * TILE, kb_last = (blk_hi / TILE) * TILE;
         // Two register sets: while tile t is computed from LDS, tile t+1 waits in one set (its loads were
         // issued an iteration ago) and the loads of tile t+2 are issued into the other.  The block-table
-        // window is loaded outside the pipelined loop, once per 64 pages.
-        const int window_keys = SIA_WAVE << ps_log2;
-        for (int w_first = kb_first; w_first <= kb_last; w_first += window_keys) {
-            const int w_last = min(kb_last, w_first + window_keys - TILE);
+        // window (64 entries from the page of the first tile it serves) is loaded outside the pipelined loop.
+        for (int w_first = kb_first, w_end; w_first <= kb_last; w_first = w_end) {
+            const int first_page = w_first >> ps_log2;
+            w_end = (first_page + SIA_WAVE) << ps_log2;  // first key beyond the window, a multiple of TILE
+            const int w_last = min(kb_last, w_end - TILE);
             PageWindow pages;
-            pages_load(pages, table, table_width, w_first >> ps_log2, lane);
+            pages_load(pages, table, table_width, first_page, lane);
             TileRegs regs_a, regs_b;
 // One tile step: issue the loads of tile kb + 2 tiles into FREE, compute tile kb from LDS stage STAGE,
 // write the tile that waits in NEXT into the other stage.  (A macro, not a lambda: register sets that a
@@ -618,27 +613,24 @@ static int log2_exact(int v) {
 SIA_EXPORT int sia_attn_mfma_head_dim() { return HD; }
 
 // Sequences 0 .. n_seqs-1 of the step, each with exactly one new token, which is row s of q (cu_q[s] = s).
-// ws_acc holds
-// n_seqs * n_heads * max_splits * head_dim floats and ws_ml twice n_seqs * n_heads * max_splits;
-// max_splits * split_keys must cover the longest sequence; split_keys is a multiple of 128.
+// n_splits workgroups share the keys of each (sequence, kv head); ws_acc holds n_seqs * n_heads * n_splits *
+// head_dim floats, ws_ml n_seqs * n_heads * n_splits * 2.
 SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                                const int* block_table, int table_width, const int* cu_q, const int* kv_len,
                                void* out, float* ws_acc, float* ws_ml, int n_seqs, int n_heads, int n_kv,
-                               int page_size, float scale, int window, int split_keys, int max_splits,
-                               hipStream_t stream) {
+                               int page_size, float scale, int window, int n_splits, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     const int ps_log2 = log2_exact(page_size);
-    if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || split_keys % (DEC_WAVES * TILE) ||
-        split_keys <= 0 || max_splits <= 0 || n_kv > 65535 || n_seqs > 65535 || q_row_stride % 8 || table_width <= 0)
+    if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || n_splits <= 0 || n_splits > 65535 ||
+        n_kv > 65535 || n_seqs > 65535 || q_row_stride % 8 || table_width <= 0)
         return SIA_BAD_ARGUMENT;
     const size_t lds_bytes = (size_t)DEC_WAVES * (n_heads / n_kv) * (HD + 2) * sizeof(float);
     if (lds_bytes > 64 * 1024) return SIA_BAD_ARGUMENT;
-    hipLaunchKernelGGL(attn_decode_kernel, dim3(max_splits, n_kv, n_seqs), dim3(DEC_WAVES * SIA_WAVE), lds_bytes,
+    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_splits, n_kv, n_seqs), dim3(DEC_WAVES * SIA_WAVE), lds_bytes,
                        stream, (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
-                       block_table, table_width, cu_q, kv_len, ws_acc, ws_ml, n_heads, n_kv, ps_log2, scale, window,
-                       split_keys, max_splits);
+                       block_table, table_width, cu_q, kv_len, ws_acc, ws_ml, n_heads, n_kv, ps_log2, scale, window);
     hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_heads, n_seqs), dim3(SIA_WAVE), 0, stream, ws_acc, ws_ml,
-                       cu_q, kv_len, (bf16_t*)out, n_heads, window, split_keys, max_splits);
+                       cu_q, (bf16_t*)out, n_heads, n_splits);
     return SIA_LAUNCH_CHECK();
 }
 

@@ -42,7 +42,7 @@ _SIGNATURES = {
 
 _ATTN_SIGNATURES = {
     "sia_attn_decode": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr],
+                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_attn_prefill": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "sia_attn_prefill_rows": [],
@@ -295,14 +295,15 @@ class HipKernels:
         return out
 
     @staticmethod
-    def decode_split(n_seqs: int, n_kv_heads: int, kv_bound: int):
-        """(keys per split, number of splits).  A split is one workgroup of four waves, and a compute
-        unit holds two of them: the smallest split whose workgroups all run at once is taken (more,
-        shorter workgroups hide latency better), and 1024 keys when even that many do not."""
-        for keys in (256, 512, 1024):
-            if n_seqs * n_kv_heads * (-(-kv_bound // keys)) <= 512:
-                return keys, -(-kv_bound // keys)
-        return 1024, -(-kv_bound // 1024)
+    def decode_split(n_seqs: int, n_kv_heads: int, kv_bound: int) -> int:
+        """Number of workgroups (four waves each) that share the keys of one (sequence, kv head).  The
+        kernel deals a sequence's tiles of 32 keys evenly to the waves.  Enough splits are taken to give
+        each of the 256 compute units a workgroup, but no more than leave every wave about four tiles at
+        the longest length the step can hold: measured at 2,304 keys, more and shorter workgroups cost
+        more in start-up and in combining than they gain."""
+        want = -(-256 // max(1, n_seqs * n_kv_heads))
+        most = max(1, kv_bound // (4 * 4 * 32))
+        return max(1, min(want, most))
 
     def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
         lib = self._attn_lib(head_dim)
@@ -312,13 +313,13 @@ class HipKernels:
         n_dec = ctx.n_decode_seqs if group <= 16 and 4 * group * (head_dim + 2) * 4 <= 65536 else 0
         if n_dec:
             bound = ctx.kv_bound or ctx.max_kv_len
-            split_keys, max_splits = self.decode_split(n_dec, n_kv_heads, bound)
-            ws_acc = torch.empty((n_dec * n_heads * max_splits * head_dim,), dtype=torch.float32, device=qkv.device)
-            ws_ml = torch.empty((n_dec * n_heads * max_splits * 2,), dtype=torch.float32, device=qkv.device)
+            n_splits = self.decode_split(n_dec, n_kv_heads, bound)
+            ws_acc = torch.empty((n_dec * n_heads * n_splits * head_dim,), dtype=torch.float32, device=qkv.device)
+            ws_ml = torch.empty((n_dec * n_heads * n_splits * 2,), dtype=torch.float32, device=qkv.device)
             self._check(lib.sia_attn_decode(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), _ptr(ws_acc), _ptr(ws_ml), n_dec, n_heads,
-                n_kv_heads, cache.page_size, float(scale), window, split_keys, max_splits, self._stream()),
+                n_kv_heads, cache.page_size, float(scale), window, n_splits, self._stream()),
                 "attn_decode")
         if n_dec < ctx.n_seqs:
             rows = lib.sia_attn_prefill_rows()
