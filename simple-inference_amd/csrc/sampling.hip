@@ -176,6 +176,90 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Argmax of every row (steps whose requests are all greedy), spread over the chip: ARGMAX_CHUNKS workgroups a
+// row each reduce a contiguous piece of it, with 16-byte loads where the row length allows, to one (value,
+// index) pair; a second kernel reduces a row's pairs.  Ties go to the lowest index, as in sample_kernel.
+// ---------------------------------------------------------------------------------------------------
+#define ARGMAX_CHUNKS 64
+#define ARGMAX_THREADS 256
+
+__device__ __forceinline__ void take_better(float& bv, int& bi, float v, int i) {
+    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+}
+
+__device__ __forceinline__ void block_argmax(float& bv, int& bi, float* vals, int* idxs) {
+#pragma unroll
+    for (int off = SIA_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, SIA_WAVE);
+        const int oi = __shfl_xor(bi, off, SIA_WAVE);
+        take_better(bv, bi, ov, oi);
+    }
+    const int wave = threadIdx.x / SIA_WAVE, n_waves = blockDim.x / SIA_WAVE;
+    if (threadIdx.x % SIA_WAVE == 0) { vals[wave] = bv; idxs[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0)
+        for (int w = 1; w < n_waves; ++w) take_better(bv, bi, vals[w], idxs[w]);
+}
+
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_chunks_kernel(const float* __restrict__ logits, int vocab,
+                                                                       float* __restrict__ ws_val,
+                                                                       int* __restrict__ ws_idx) {
+    __shared__ float vals[ARGMAX_THREADS / SIA_WAVE];
+    __shared__ int idxs[ARGMAX_THREADS / SIA_WAVE];
+    const int chunk = blockIdx.x, r = blockIdx.y;
+    const float* row = logits + (size_t)r * vocab;
+    float bv = -INFINITY;
+    int bi = vocab;
+    if (vocab % 4 == 0) {
+        const int quads = vocab / 4, per = (quads + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+        const int q_end = min(quads, (chunk + 1) * per);
+        for (int q = chunk * per + threadIdx.x; q < q_end; q += ARGMAX_THREADS) {
+            const float4 v = reinterpret_cast<const float4*>(row)[q];
+            take_better(bv, bi, v.x, 4 * q);
+            take_better(bv, bi, v.y, 4 * q + 1);
+            take_better(bv, bi, v.z, 4 * q + 2);
+            take_better(bv, bi, v.w, 4 * q + 3);
+        }
+    } else {
+        const int per = (vocab + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+        const int i_end = min(vocab, (chunk + 1) * per);
+        for (int i = chunk * per + threadIdx.x; i < i_end; i += ARGMAX_THREADS) take_better(bv, bi, row[i], i);
+    }
+    block_argmax(bv, bi, vals, idxs);
+    if (threadIdx.x == 0) {
+        ws_val[r * ARGMAX_CHUNKS + chunk] = bv;
+        ws_idx[r * ARGMAX_CHUNKS + chunk] = bi;
+    }
+}
+
+__global__ __launch_bounds__(SIA_WAVE) void argmax_finish_kernel(const float* __restrict__ ws_val,
+                                                                 const int* __restrict__ ws_idx,
+                                                                 int* __restrict__ out, int vocab) {
+    __shared__ float vals[1];
+    __shared__ int idxs[1];
+    const int r = blockIdx.x;
+    float bv = -INFINITY;
+    int bi = vocab;
+    for (int c = threadIdx.x; c < ARGMAX_CHUNKS; c += SIA_WAVE)
+        take_better(bv, bi, ws_val[r * ARGMAX_CHUNKS + c], ws_idx[r * ARGMAX_CHUNKS + c]);
+    block_argmax(bv, bi, vals, idxs);
+    if (threadIdx.x == 0) out[r] = bi < vocab ? bi : 0;
+}
+
+SIA_EXPORT int sia_argmax_workspace_per_row() { return ARGMAX_CHUNKS; }
+
+// ws_val and ws_idx hold rows * sia_argmax_workspace_per_row() elements each.
+SIA_EXPORT int sia_argmax(const float* logits, int* out, float* ws_val, int* ws_idx, int rows, int vocab,
+                          hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0 || rows > 65535) return SIA_BAD_ARGUMENT;
+    hipLaunchKernelGGL(argmax_chunks_kernel, dim3(ARGMAX_CHUNKS, rows), dim3(ARGMAX_THREADS), 0, stream, logits,
+                       vocab, ws_val, ws_idx);
+    hipLaunchKernelGGL(argmax_finish_kernel, dim3(rows), dim3(SIA_WAVE), 0, stream, ws_val, ws_idx, out, vocab);
+    return SIA_LAUNCH_CHECK();
+}
+
 SIA_EXPORT int sia_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
                           const float* uniform, int* out, int rows, int vocab, hipStream_t stream) {
     if (rows <= 0) return 0;

@@ -34,6 +34,8 @@ _SIGNATURES = {
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_sample": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "sia_argmax": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "sia_argmax_workspace_per_row": [],
     "sia_gemm_skinny": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_gemm_skinny_max_rows": [],
     "sia_gemm_skinny_swiglu": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -330,9 +332,19 @@ class HipKernels:
                 cache.page_size, float(scale), window, self._stream()), "attn_prefill")
 
     # -- sampling ------------------------------------------------------------------
-    def sample(self, logits, temperature, top_k, top_p, uniform):
+    def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False):
+        """One token per row.  ``all_greedy`` (every temperature is 0, which the caller knows on the host)
+        takes the argmax kernels that spread a row over the chip."""
         rows, vocab = logits.shape
         self._want(logits, "logits", torch.float32)
+        if all_greedy:
+            out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+            per_row = self.core.sia_argmax_workspace_per_row()
+            ws_val = torch.empty((rows * per_row,), dtype=torch.float32, device=logits.device)
+            ws_idx = torch.empty((rows * per_row,), dtype=torch.int32, device=logits.device)
+            self._check(self.core.sia_argmax(_ptr(logits), _ptr(out), _ptr(ws_val), _ptr(ws_idx), rows, vocab,
+                                             self._stream()), "argmax")
+            return out
         self._want(temperature, "temperature", torch.float32, (rows,))
         self._want(top_k, "top_k", torch.int32, (rows,))
         self._want(top_p, "top_p", torch.float32, (rows,))

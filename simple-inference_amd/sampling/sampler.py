@@ -30,4 +30,5 @@ class Sampler:
             host[2, i] = 0.0 if p.greedy else uniform_for(p.seed, n)
         top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32)
         dev = host.to(self.device)
-        return self.kernels.sample(logits, dev[0], top_k.to(self.device), dev[1], dev[2])
+        return self.kernels.sample(logits, dev[0], top_k.to(self.device), dev[1], dev[2],
+                                   all_greedy=all(p.greedy for p in params))

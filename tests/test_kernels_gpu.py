@@ -285,6 +285,23 @@ def test_sample_matches_twin(hip, vocab):
         assert got.tolist() == ref.tolist(), (seed, got.tolist(), ref.tolist())
 
 
+@pytest.mark.parametrize("vocab", [5, 1001, 4096, 128256])
+def test_argmax_over_the_chip_matches_the_one_workgroup_argmax(hip, vocab):
+    rows = 9
+    logits = rnd(rows, vocab, seed=3, scale=3.0)
+    logits[1] = 0.0                                   # all equal: index 0
+    logits[2, vocab - 1] = 50.0                       # the last element
+    logits[3, [vocab // 2, vocab - 2 if vocab > 2 else 0]] = 60.0   # a tie across chunks: the lower index
+    z = lambda dt, v: torch.full((rows,), v, dtype=dt, device=DEV)
+    args = (logits, z(torch.float32, 0.0), z(torch.int32, 0), z(torch.float32, 1.0), z(torch.float32, 0.5))
+    spread = hip.sample(*args, all_greedy=True)
+    assert spread.tolist() == hip.sample(*args).tolist()
+    library = torch.argmax(logits, -1).tolist()
+    assert [t for i, t in enumerate(spread.tolist()) if i not in (1, 3)] == [t for i, t in enumerate(library) if i not in (1, 3)]
+    assert spread[1].item() == 0 and spread[2].item() == vocab - 1
+    assert spread[3].item() == min(vocab // 2, vocab - 2 if vocab > 2 else 0)
+
+
 def test_sample_greedy_is_argmax_with_lowest_index_on_ties(hip):
     logits = torch.zeros(3, 5000, device=DEV)
     logits[0, 4321] = 1.0

@@ -114,7 +114,7 @@ class TwinKernels:
         return out.view(N, n_heads * head_dim).to(qkv.dtype)
 
     # -- sampling --------------------------------------------------------------
-    def sample(self, logits, temperature, top_k, top_p, uniform):
+    def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False):
         out = []
         for r in range(logits.shape[0]):
             row = logits[r].double()
