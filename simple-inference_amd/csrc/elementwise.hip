@@ -153,16 +153,42 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     out[(size_t)n * inter + i] = from_float<T>(g / (1.f + expf(-g)) * u);
 }
 
+// Eight elements a thread, 16- or 32-byte accesses (inter % 8 == 0).
+template <typename T>
+__global__ void swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
+    const int n = blockIdx.y;
+    const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (i >= inter) return;
+    const T* row = gu + (size_t)n * 2 * inter;
+    Vec8<T> vg, vu;
+    vg.load(row + i);
+    vu.load(row + inter + i);
+    float g[8], u[8];
+    vg.get(g);
+    vu.get(u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) g[j] = g[j] / (1.f + expf(-g[j])) * u[j];
+    vg.set(g);
+    vg.store(out + (size_t)n * inter + i);
+}
+
 SIA_EXPORT int sia_swiglu(const void* gu, void* out, int n_tokens, int inter, int dtype, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (n_tokens > 65535) return SIA_BAD_ARGUMENT;
+    if (dtype != SIA_F32 && dtype != SIA_BF16) return SIA_BAD_ARGUMENT;
+    if (inter % 8 == 0) {
+        dim3 block(256), grid((inter / 8 + 255) / 256, n_tokens);
+        if (dtype == SIA_F32)
+            hipLaunchKernelGGL(swiglu_vec_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)out, inter);
+        else
+            hipLaunchKernelGGL(swiglu_vec_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)out, inter);
+        return SIA_LAUNCH_CHECK();
+    }
     dim3 block(256), grid((inter + 255) / 256, n_tokens);
     if (dtype == SIA_F32)
         hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)out, inter);
-    else if (dtype == SIA_BF16)
-        hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)out, inter);
     else
-        return SIA_BAD_ARGUMENT;
+        hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)out, inter);
     return SIA_LAUNCH_CHECK();
 }
 

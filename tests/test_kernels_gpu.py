@@ -102,7 +102,7 @@ def test_rmsnorm_eps_is_inside_the_root(hip):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("inter", [24, 1000, 8192])
+@pytest.mark.parametrize("inter", [24, 37, 1000, 8192])
 def test_swiglu(hip, dtype, inter):
     gu = rnd(5, 2 * inter, dtype=dtype, scale=3.0)
     torch.testing.assert_close(hip.swiglu(gu).float(), twin.swiglu(gu).float(), **tol(dtype))
