@@ -64,6 +64,26 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 constexpr float LOG2E = 1.4426950408889634f;
 
+// Maximum and sum over the four lanes r, r+16, r+32, r+48 that share a q column, for every lane, by the
+// register swaps between the wave's rows of 16 lanes (no trip through LDS as a general lane shuffle makes):
+// v_permlane16_swap exchanges rows 1, 3 of its first operand with rows 0, 2 of its second, v_permlane32_swap
+// the upper half of the first with the lower half of the second; either way the two results hold, lane by
+// lane, the two values to combine.  The sum is (row 0 + row 1) + (row 2 + row 3) in every lane.
+__device__ __forceinline__ float column_max(float v) {
+    uint32_t u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    u = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+    const auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float column_sum(float v) {
+    uint32_t u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    u = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // 64 consecutive entries of a sequence's block table, one per lane.
 struct PageWindow {
     int base;  // index of the entry that lane 0 holds
@@ -142,8 +162,7 @@ __device__ __forceinline__ void softmax_update(floatx4 (&s)[NQ][2], int kb, cons
         }
         float mx = fmaxf(fmaxf(fmaxf(s[n][0][0], s[n][0][1]), fmaxf(s[n][0][2], s[n][0][3])),
                          fmaxf(fmaxf(s[n][1][0], s[n][1][1]), fmaxf(s[n][1][2], s[n][1][3])));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, SIA_WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, SIA_WAVE));
+        mx = column_max(mx);
         const float m_new = fmaxf(m[n], mx * scale_log2);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
         const float alpha = fast_exp2(m[n] - m_use);
@@ -156,8 +175,7 @@ __device__ __forceinline__ void softmax_update(floatx4 (&s)[NQ][2], int kb, cons
                 s[n][h][i] = e;
                 sum += e;
             }
-        sum += __shfl_xor(sum, 16, SIA_WAVE);
-        sum += __shfl_xor(sum, 32, SIA_WAVE);
+        sum = column_sum(sum);
         l[n] = l[n] * alpha + sum;
         m[n] = m_new;
         if (__any(alpha != 1.f)) {
@@ -379,29 +397,32 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
 // ---------------------------------------------------------------------------------------------------
 // prefill: runs of several tokens (works for single tokens too, without splitting the keys)
 // ---------------------------------------------------------------------------------------------------
-constexpr int PF_NQ = HD <= 128 ? 2 : 1;        // groups of 16 tokens per wave
-constexpr int PF_WAVES = 4;
-constexpr int PF_ROWS = PF_WAVES * PF_NQ * 16;  // tokens per workgroup
-constexpr int PF_THREADS = PF_WAVES * SIA_WAVE;
+// Two shapes of workgroup, both of PF_ROWS tokens: 4 waves of 32 tokens each (fewer reads from LDS per MFMA:
+// the faster one when there are workgroups enough to keep two on every compute unit), and 8 waves of 16
+// tokens each (two waves a SIMD from the start, so that one's softmax runs beside the other's MFMAs: the
+// faster one for short prompts and portions).  Head sizes above 128 take 4 waves of 16 tokens.
+constexpr int PF_ROWS = HD <= 128 ? 128 : 64;  // tokens per workgroup
 // Key and value tiles are shared by the workgroup's waves through LDS (two stages).  Rows are padded by
 // 16 bytes so that the 16 lanes of a 128-bit read hit 64 different banks.
 constexpr int K_STRIDE = HD + 8;                // elements per key row
 constexpr int V_STRIDE = TILE + 8;              // elements per dim row (32 positions + pad)
-constexpr int K_CHUNKS = TILE * HD / 8;         // 16-byte pieces of a key tile
-constexpr int PF_PER_THREAD = (K_CHUNKS + PF_THREADS - 1) / PF_THREADS;
+constexpr int K_CHUNKS = TILE * HD / 8;         // 16-byte pieces of a key tile (a value tile has as many)
 constexpr bool PF_USE_LDS = (2 * (TILE * K_STRIDE + HD * V_STRIDE) * 2) <= 64 * 1024;
 
-// What one thread carries from global memory to LDS for one tile.
+// What one thread of a workgroup of TEAM threads carries from global memory to LDS for one tile.
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;  // a plain 16-byte register value
+template <int TEAM>
 struct TileRegs {
-    u32x4 k[PF_PER_THREAD];
-    u32x4 v[PF_PER_THREAD];
+    static constexpr int PER_THREAD = (K_CHUNKS + TEAM - 1) / TEAM;
+    u32x4 k[PER_THREAD];
+    u32x4 v[PER_THREAD];
 };
 
 // Issues the global loads of the tile at kb.  Key chunk c is (key c / (HD/8), dims 8 (c % (HD/8)) ..);
 // value chunks are ordered (page segment, dim, group of 8 positions), so that consecutive threads read
 // consecutive 16 bytes of a page.  Keys outside [lo, hi] are clamped into it (see load_stage).
-__device__ __forceinline__ void tile_fetch(TileRegs& t, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
+template <int TEAM>
+__device__ __forceinline__ void tile_fetch(TileRegs<TEAM>& t, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
                                            const PageWindow& pages, int ps_log2, int n_kv, int hk, int kb, int lo,
                                            int hi) {
     const int ps = 1 << ps_log2;
@@ -409,9 +430,9 @@ __device__ __forceinline__ void tile_fetch(TileRegs& t, const bf16_t* __restrict
     const int seg_keys = min(ps, TILE);            // positions of one page inside a tile
     const int seg_chunks = HD * (seg_keys / 8);    // 16-byte pieces of one page's values inside a tile
 #pragma unroll
-    for (int i = 0; i < PF_PER_THREAD; ++i) {
-        const int c = threadIdx.x + i * PF_THREADS;
-        if (K_CHUNKS % PF_THREADS != 0 && c >= K_CHUNKS) break;
+    for (int i = 0; i < TileRegs<TEAM>::PER_THREAD; ++i) {
+        const int c = threadIdx.x + i * TEAM;
+        if (K_CHUNKS % TEAM != 0 && c >= K_CHUNKS) break;
         {
             const int key = min(max(kb + c / (HD / 8), t_lo), t_hi);
             const int page = pages_get(pages, key >> ps_log2);
@@ -430,15 +451,16 @@ __device__ __forceinline__ void tile_fetch(TileRegs& t, const bf16_t* __restrict
 
 // Writes a fetched tile into an LDS stage.  Key rows are stored in the order the score MFMAs read them
 // (row 16h + m holds key 8(m/4) + 4h + m%4), so that the 16 lanes of a read take 16 consecutive rows.
-__device__ __forceinline__ void tile_store(const TileRegs& t, bf16_t* __restrict__ k_lds, bf16_t* __restrict__ v_lds,
+template <int TEAM>
+__device__ __forceinline__ void tile_store(const TileRegs<TEAM>& t, bf16_t* __restrict__ k_lds, bf16_t* __restrict__ v_lds,
                                            int ps_log2) {
     const int ps = 1 << ps_log2;
     const int seg_keys = min(ps, TILE);
     const int seg_chunks = HD * (seg_keys / 8);
 #pragma unroll
-    for (int i = 0; i < PF_PER_THREAD; ++i) {
-        const int c = threadIdx.x + i * PF_THREADS;
-        if (K_CHUNKS % PF_THREADS != 0 && c >= K_CHUNKS) break;
+    for (int i = 0; i < TileRegs<TEAM>::PER_THREAD; ++i) {
+        const int c = threadIdx.x + i * TEAM;
+        if (K_CHUNKS % TEAM != 0 && c >= K_CHUNKS) break;
         const int key = c / (HD / 8);
         const int row = ((key >> 2) & 1) * 16 + (key >> 3) * 4 + (key & 3);
         *reinterpret_cast<u32x4*>(k_lds + row * K_STRIDE + (c % (HD / 8)) * 8) = t.k[i];
@@ -483,7 +505,9 @@ __device__ __forceinline__ void compute_from_lds(const bf16_t* __restrict__ k_ld
     }
 }
 
-__global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
+// PF_NQ groups of 16 tokens per wave, PF_WAVES waves: PF_NQ * PF_WAVES * 16 = PF_ROWS.
+template <int PF_NQ, int PF_WAVES>
+__global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale,
@@ -553,7 +577,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
             const int w_last = min(kb_last, w_end - TILE);
             PageWindow pages;
             pages_load(pages, table, table_width, first_page, lane);
-            TileRegs regs_a, regs_b;
+            TileRegs<PF_WAVES * SIA_WAVE> regs_a, regs_b;
 // One tile step: issue the loads of tile kb + 2 tiles into FREE, compute tile kb from LDS stage STAGE,
 // write the tile that waits in NEXT into the other stage.  (A macro, not a lambda: register sets that a
 // closure captures by reference end up in scratch memory.)
@@ -645,9 +669,19 @@ SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_p
     const int ps_log2 = log2_exact(page_size);
     if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads > 65535 || q_row_stride % 8 || table_width <= 0)
         return SIA_BAD_ARGUMENT;
-    hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_tiles, n_heads), dim3(PF_WAVES * SIA_WAVE), 0, stream,
-                       (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table,
-                       table_width, cu_q, kv_len, (bf16_t*)out, n_heads, n_kv, ps_log2, scale, window, seq_begin,
-                       seq_end);
+#define LAUNCH(NQ, WAVES)                                                                                       \
+    hipLaunchKernelGGL((attn_prefill_kernel<NQ, WAVES>), dim3(n_tiles, n_heads), dim3(WAVES * SIA_WAVE), 0, stream,  \
+                       (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, \
+                       table_width, cu_q, kv_len, (bf16_t*)out, n_heads, n_kv, ps_log2, scale, window, seq_begin,  \
+                       seq_end)
+    if constexpr (HD > 128) {
+        LAUNCH(1, PF_ROWS / 16);
+    } else {
+        if ((long long)n_tiles * n_heads <= 2 * 256)  // not two workgroups for each of the 256 compute units
+            LAUNCH(1, PF_ROWS / 16);
+        else
+            LAUNCH(2, PF_ROWS / 32);
+    }
+#undef LAUNCH
     return SIA_LAUNCH_CHECK();
 }
