@@ -1,9 +1,10 @@
 """The engine: requests in, tokens out (reference: ``serving/engine.py:95-517``).
 
-``add_request`` queues a request; ``step`` runs one iteration: finished requests leave, waiting
-ones are admitted while slots, token budget and pages allow, the scheduler picks this step's
-tokens (one per decoding request, then prompt portions), ONE call of the step function runs
-them all as one batch, and the sampler turns the returned logits into tokens.  ``run`` steps
+``add_request`` queues a request; ``step`` runs one iteration: finished requests leave, the
+scheduler picks this step's tokens (one per decoding request, then prompt portions) and admits
+waiting requests into the room that is left while slots, token budget and pages allow, ONE call
+of the step function runs them all as one batch, and the sampler turns the returned logits into
+tokens.  ``run`` steps
 until nothing is left.  The reference's step runs two forwards instead, one for whole prompts
 and one for decoded tokens (``serving/engine.py:330-349``).
 """
@@ -119,6 +120,8 @@ class Engine:
         shared: List[int] = []
         if self.prefix_cache is not None:
             shared = self.prefix_cache.match(req.prompt_tokens)
+            if self._prefix_still_being_written(req, len(shared)):
+                return False
             need = self.cache.groups[0].pages_to_reserve(total, self.cfg.chunk_tokens) - len(shared)
             if not self.prefix_cache.evict_until_available(need, protected=set(shared)):
                 return False
@@ -129,13 +132,32 @@ class Engine:
         req.num_computed = req.cached_prefix_len
         return True
 
+    def _prefix_still_being_written(self, req: Request, matched_pages: int) -> bool:
+        """True if a request that is still running its prompt shares more whole pages with ``req`` than the
+        prefix cache holds yet: ``req`` then waits the few steps until they are written, instead of
+        computing them a second time."""
+        ps = self.cfg.block_size
+        reusable = (req.prompt_len - 1) // ps
+        if matched_pages >= reusable:
+            return False
+        for other in self.scheduler.running:
+            if other.state is not RequestState.PREFILL:
+                continue
+            limit = min(reusable, other.prompt_len // ps)
+            pages = matched_pages
+            while pages < limit and req.prompt_tokens[pages * ps:(pages + 1) * ps] == \
+                    other.prompt_tokens[pages * ps:(pages + 1) * ps]:
+                pages += 1
+            if pages > matched_pages and req.prompt_tokens[:matched_pages * ps] == other.prompt_tokens[:matched_pages * ps]:
+                return True
+        return False
+
     # -- one iteration ---------------------------------------------------------------
     @torch.no_grad()
     def step(self) -> Dict[int, int]:
         """Runs one iteration; returns {request id: token} for every request that emitted one."""
         self.scheduler.evict_finished()
-        self.scheduler.admit(self._try_admit)
-        plan = self.scheduler.plan_step()
+        plan = self.scheduler.plan_step(self._try_admit)   # admits, too: into steps with room for prompt tokens
         if not plan:
             return {}
         entries, emitters = [], []
@@ -160,6 +182,9 @@ class Engine:
             logits = self.runner.run(entries)
         for req, n in plan:
             req.num_computed += n
+            if self.prefix_cache is not None and req.state is RequestState.PREFILL and req.num_computed < req.prompt_len:
+                # pages a prompt has filled so far can be shared from the next step on
+                self.prefix_cache.insert(req.prompt_tokens[:req.num_computed], self.cache.table(0, req.id))
         emitted: Dict[int, int] = {}
         if emitters:
             tokens = self.sampler.sample(logits, [r.params for r in emitters], [r.num_generated for r in emitters])

@@ -13,6 +13,11 @@ What the reference lacks is the cut of prompts into portions (``plan.md:811-868`
 the prefilling requests in admission order until ``chunk_tokens`` tokens are in the step.  A
 request turns to DECODE in the step that runs its last prompt token and emits its first token
 from that step.
+
+Given the admission test, ``plan_step`` also admits: a waiting request enters only in a step
+that still has room for its first prompt tokens.  So a request is not promised pages while it
+could not run anyway, and when prompts arrive together the later ones are matched against the
+prefix cache after the earlier ones have written their pages, not before.
 """
 
 from __future__ import annotations
@@ -49,10 +54,13 @@ class Scheduler:
     def _running_tokens(self) -> int:
         return sum(r.context_len for r in self.running)
 
-    def admit(self, can_admit: Optional[Callable[[Request], bool]] = None) -> List[Request]:
+    def admit(self, can_admit: Optional[Callable[[Request], bool]] = None,
+              limit: Optional[int] = None) -> List[Request]:
+        """Admits from the head of the queue while slots, the token budget and ``can_admit`` allow, at most
+        ``limit`` requests."""
         admitted: List[Request] = []
         used = self._running_tokens()
-        while self.waiting and len(self.running) < self.max_running:
+        while self.waiting and len(self.running) < self.max_running and (limit is None or len(admitted) < limit):
             head = self.waiting[0]
             if (self.running or admitted) and used + head.prompt_len > self.token_budget:
                 break
@@ -65,8 +73,12 @@ class Scheduler:
             used += head.prompt_len
         return admitted
 
-    def plan_step(self) -> List[Tuple[Request, int]]:
-        """(request, number of its next tokens) for one step: decoded tokens, then prompt portions."""
+    def plan_step(self, can_admit: Optional[Callable[[Request], bool]] = None,
+                  admit: bool = False) -> List[Tuple[Request, int]]:
+        """(request, number of its next tokens) for one step: decoded tokens, then prompt portions.
+
+        With ``admit`` (or an admission test), waiting requests are admitted one by one while the step
+        has room left for prompt tokens, and get their first portion in this step."""
         plan: List[Tuple[Request, int]] = []
         room = self.chunk_tokens
         for r in self.running:
@@ -77,6 +89,15 @@ class Scheduler:
             if r.state is RequestState.PREFILL:
                 if room <= 0:
                     break
+                n = min(room, r.prompt_len - r.num_computed)
+                plan.append((r, n))
+                room -= n
+        if admit or can_admit is not None:
+            while room > 0:
+                newcomers = self.admit(can_admit, limit=1)
+                if not newcomers:
+                    break
+                r = newcomers[0]
                 n = min(room, r.prompt_len - r.num_computed)
                 plan.append((r, n))
                 room -= n

@@ -87,3 +87,30 @@ def test_engine_with_prefix_reuse_gives_the_same_tokens(tmp_path):
     eng.cache.check()
     eng.reset()
     assert eng.cache.free_pages() == 24
+
+
+def test_prompts_that_arrive_together_share_what_the_first_of_them_wrote(tmp_path):
+    """Several prompts with one long prefix are queued at once.  Requests enter a step only when it has room
+    for their tokens, and a prompt's filled pages are cached step by step: so the later ones find the prefix,
+    run their own ends only and generate what they generate without the cache."""
+    tiny = TINIES["a"]
+    folder = write_tiny_model(tmp_path, tiny, seed=62)
+    prefix = random_tokens(tiny.config["vocab_size"], 44, seed=3)
+    prompts = [prefix + random_tokens(tiny.config["vocab_size"], 3 + i, seed=10 + i) for i in range(5)]
+
+    def run(use):
+        eng = Engine.from_folder(folder, EngineConfig(
+            device="cpu", dtype="float32", max_seq_len=96, block_size=4, max_running=4, chunk_tokens=16, eos_id=-1,
+            num_kv_blocks=120, use_prefix_cache=use), TwinKernels())
+        reqs = [eng.add_request(p, max_new_tokens=5) for p in prompts]
+        eng.run()
+        eng.cache.check()
+        return eng, reqs
+    _, plain_reqs = run(False)
+    eng, reqs = run(True)
+    assert [r.generated for r in reqs] == [r.generated for r in plain_reqs]
+    assert reqs[0].cached_prefix_len == 0
+    assert all(r.cached_prefix_len == 44 for r in reqs[1:])      # 11 whole pages of 4
+    assert eng.stats["prefill_tokens"] == sum(len(p) for p in prompts) - 4 * 44
+    eng.reset()
+    assert eng.cache.free_pages() == 120

@@ -55,6 +55,25 @@ def test_plan_gives_decoders_one_token_then_prompt_portions_in_order():
     assert [(r.id, n) for r, n in s.plan_step()] == [(d1.id, 1), (p1.id, 1), (d2.id, 1), (p2.id, 3)]
 
 
+def test_plan_admits_newcomers_only_into_room_for_their_first_tokens():
+    s = Scheduler(max_running=4, token_budget=1000, chunk_tokens=8)
+    a, b, c, d = req(11), req(3), req(6), req(2)
+    for r in (a, b, c, d):
+        s.add(r)
+    plan = s.plan_step(admit=True)
+    assert [(r.id, n) for r, n in plan] == [(a.id, 8)]          # a fills the step: nobody else enters yet
+    assert [r.state for r in (a, b, c)] == [RequestState.PREFILL, RequestState.WAITING, RequestState.WAITING]
+    a.num_computed = 8
+    plan = s.plan_step(admit=True)                               # a's rest, all of b, the start of c
+    assert [(r.id, n) for r, n in plan] == [(a.id, 3), (b.id, 3), (c.id, 2)]
+    assert d.state is RequestState.WAITING and len(s.running) == 3
+    # the admission test still decides, and nobody overtakes the head of the queue
+    a.num_computed, b.num_computed, c.num_computed = 11, 3, 6
+    a.state = b.state = c.state = RequestState.DECODE
+    assert [(r.id, n) for r, n in s.plan_step(lambda r: False)] == [(a.id, 1), (b.id, 1), (c.id, 1)]
+    assert [(r.id, n) for r, n in s.plan_step(lambda r: True)] == [(a.id, 1), (b.id, 1), (c.id, 1), (d.id, 2)]
+
+
 # ---- the engine on the CPU -----------------------------------------------------------------------
 @pytest.fixture(scope="module")
 def folder(tmp_path_factory):
