@@ -10,6 +10,12 @@ step function over the batch, sampling).  The default run has the layer sizes of
 headline it reports the prefill of one 2,048-token prompt, decode at batch 1 and 64, and how
 close the decode step comes to the HBM roofline and the prefill to the matrix-core peak.
 
+Two further workloads run whole request streams through the scheduler (``--workload``):
+``continuous``: 128 requests at the 1B shape, prompts of 64..2,048 and outputs of 32..512 tokens,
+prompts cut into portions of 512; ``shared-prefix``: 64 requests at the 8B shape with one
+1,024-token prefix, 256 tokens of their own and 256 decoded tokens each, with and without
+prefix reuse.  They print one JSON line of their own kind.
+
 The engine runs on one GPU; asked for more it says so and exits with 2.
 """
 
@@ -42,6 +48,8 @@ def parse_args(argv=None):
     ap.add_argument("--points", default="1,64", help="further decode batch sizes to report, comma separated")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix"])
+    ap.add_argument("--max-running", type=int, default=64, help="request slots of the stream workloads")
     return ap.parse_args(argv)
 
 
@@ -121,6 +129,63 @@ def measure_prefill(engine, tokens, repeats=3, seed=100):
     return best
 
 
+def run_stream(preset_name, requests, max_running, max_seq_len, prefix_cache, args):
+    """Queues all requests at once and steps the engine dry; returns the figures of the run."""
+    from simple_inference_amd import Engine, EngineConfig, SamplingParams, preset
+
+    ecfg = EngineConfig(max_running=max_running, max_seq_len=max_seq_len, chunk_tokens=512, dtype=args.dtype,
+                        eos_id=-1, use_graphs=not args.no_graphs, use_prefix_cache=prefix_cache, device="cuda:0")
+    engine = Engine.from_random(preset(preset_name), seed=args.seed, engine_cfg=ecfg, std=0.02,
+                                generate_on_device=True)
+    handles = [engine.add_request(p, params=SamplingParams(temperature=0.0, max_new_tokens=n, ignore_eos=True))
+               for p, n in requests]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while engine.has_work():
+        engine.step()
+    torch.cuda.synchronize()
+    sec = time.perf_counter() - t0
+    assert all(len(h.generated) == n for h, (_, n) in zip(handles, requests))
+    engine.cache.check()
+    out = {"seconds": round(sec, 3), "steps": engine.stats["steps"], "prompt_tokens": sum(len(p) for p, _ in requests),
+           "prefill_tokens_run": engine.stats["prefill_tokens"], "generated_tokens": engine.stats["decode_tokens"] + len(requests),
+           "generated_tok_s": round(sum(n for _, n in requests) / sec, 1)}
+    del engine
+    torch.cuda.empty_cache()
+    return out
+
+
+def stream_workload(args):
+    import random
+
+    from simple_inference_amd import preset
+
+    rng = random.Random(args.seed)
+    if args.workload == "continuous":
+        name = "llama-3.2-1b"
+        vocab = preset(name)["vocab_size"]
+        requests = [([rng.randrange(vocab) for _ in range(rng.randint(64, 2048))], rng.randint(32, 512))
+                    for _ in range(128)]
+        run = run_stream(name, requests, args.max_running, 4096, False, args)
+        line = {"metric": "generated tok/s, continuous batching of 128 requests (1B shape)", "value": run["generated_tok_s"],
+                "run": run}
+    else:
+        name = "llama-3.1-8b"
+        vocab = preset(name)["vocab_size"]
+        shared = [rng.randrange(vocab) for _ in range(1024)]
+        requests = [(shared + [rng.randrange(vocab) for _ in range(256)], 256) for _ in range(64)]
+        reuse = run_stream(name, requests, args.max_running, 8192, True, args)
+        plain = run_stream(name, requests, args.max_running, 8192, False, args)
+        line = {"metric": "generated tok/s, 64 requests with a shared 1,024-token prefix (8B shape), prefix reuse on",
+                "value": reuse["generated_tok_s"], "run": reuse, "without_reuse": plain}
+    line.update({"unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                 "data": "synthetic (seeded random weights N(0, 0.02) and uniform-random token ids)",
+                 "config": {"model": name + "-shape", "max_running": args.max_running, "chunk_tokens": 512,
+                            "graphs": not args.no_graphs}})
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main(argv=None):
     args = parse_args(argv)
     if args.gpus != 1:
@@ -129,6 +194,8 @@ def main(argv=None):
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
+    if args.workload != "decode":
+        return stream_workload(args)
     points = [int(p) for p in args.points.split(",") if p]
     max_batch = max([args.batch] + points)
     total_len = max(args.context + args.warmup + args.steps + max_batch + 2, args.prefill_tokens + 2)
