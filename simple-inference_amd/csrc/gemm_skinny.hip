@@ -25,24 +25,22 @@ __device__ __forceinline__ bf16x8 ld8(const bf16_t* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
 
-enum SkinnyEpilogue { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_PARTIAL = 2 };
+enum SkinnyEpilogue { EPI_STORE = 0, EPI_SWIGLU = 1 };
 
 // RB: blocks of 16 rows of W per workgroup, rb_stride rows apart; UNROLL: steps whose loads are in flight
-// together.  The workgroup covers k in [blockIdx.y * k_per_split, + k_per_split) (a multiple of 64).
+// together.
 //   EPI_STORE:   Y[m][n0 + 16 rb + n]  (TOut)
 //   EPI_SWIGLU:  RB = 2, row block 0 is the gate and row block 1 (rb_stride = intermediate size) the up
 //                projection: Y[m][n0 + n] = silu(gate) * up, in float, rounded once
-//   EPI_PARTIAL: float partial sums Y[blockIdx.y][m][n]; the consumer adds the splits in order
 template <typename TOut, int RB, int UNROLL, int EPI>
 __global__ __launch_bounds__(SK_WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                         const bf16_t* __restrict__ W,
                                                                         TOut* __restrict__ Y, int M, int N, int K,
-                                                                        int rb_stride, int k_per_split) {
+                                                                        int rb_stride) {
     __shared__ float part[SK_WAVES][RB][16][17];
     constexpr int CHUNK = SK_STEP * UNROLL;  // one wave's share of a round
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * 16 * (EPI == EPI_SWIGLU ? 1 : RB);
-    const int k_begin = blockIdx.y * k_per_split, k_end = min(K, k_begin + k_per_split);
     const bf16_t* w_row = W + (size_t)(n0 + r) * K + g * 16;
     const bf16_t* x_row = X + (size_t)min(r, M - 1) * K + g * 16;
     const bool x_live = r < M;
@@ -51,12 +49,12 @@ __global__ __launch_bounds__(SK_WAVES* SIA_WAVE) void gemm_skinny_kernel(const b
     floatx4 acc[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) acc[rb] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = k_begin + wave * CHUNK; k0 < k_end; k0 += SK_WAVES * CHUNK) {
+    for (int k0 = wave * CHUNK; k0 < K; k0 += SK_WAVES * CHUNK) {
         bf16x8 a[UNROLL][RB][2], b[UNROLL][2];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int k = k0 + u * SK_STEP;
-            const bool in = k < k_end;  // ranges are multiples of 64: a step is inside or outside as a whole
+            const bool in = k < K;  // K is a multiple of 64: a step is inside or outside as a whole
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
                 a[u][rb][0] = in ? ld8(w_row + (size_t)rb * rb_stride * K + k) : zero;
@@ -98,30 +96,12 @@ __global__ __launch_bounds__(SK_WAVES* SIA_WAVE) void gemm_skinny_kernel(const b
             float s = 0.f;
 #pragma unroll
             for (int w = 0; w < SK_WAVES; ++w) s += part[w][rb][m][n];
-            const size_t at = (size_t)m * N + n0 + rb * rb_stride + n;
-            if (EPI == EPI_PARTIAL)
-                Y[(size_t)blockIdx.y * M * N + at] = from_float<TOut>(s);
-            else
-                Y[at] = from_float<TOut>(s);
+            Y[(size_t)m * N + n0 + rb * rb_stride + n] = from_float<TOut>(s);
         }
     }
 }
 
 SIA_EXPORT int sia_gemm_skinny_max_rows() { return 16; }
-
-// How many ways K is split across workgroups for an [N, K] matrix: enough workgroups to fill the chip,
-// each split a multiple of 512 k (8 waves x 64).  Depends on N and K only, so a row's sum order does too.
-SIA_EXPORT int sia_gemm_skinny_splits(int N, int K) {
-    if (N % 16 || K % 512) return 1;
-    const int blocks = (N % 64 == 0 && N / 64 >= 256) ? N / 64 : N / 16;
-    int best = 1;
-    for (int s = 1; s <= 8; ++s) {
-        if ((K / 512) % s) continue;
-        best = s;
-        if (blocks * s >= 512) break;
-    }
-    return best;
-}
 
 template <typename TOut>
 static void launch_skinny(const bf16_t* X, const bf16_t* W, TOut* Y, int M, int N, int K, hipStream_t stream) {
@@ -129,10 +109,10 @@ static void launch_skinny(const bf16_t* X, const bf16_t* W, TOut* Y, int M, int 
     // 64 rows a workgroup when that still gives every compute unit a workgroup, else 16.
     if (N % 64 == 0 && N / 64 >= 256)
         hipLaunchKernelGGL((gemm_skinny_kernel<TOut, 4, 2, EPI_STORE>), dim3(N / 64), block, 0, stream, X, W, Y, M, N,
-                           K, 16, K);
+                           K, 16);
     else
         hipLaunchKernelGGL((gemm_skinny_kernel<TOut, 1, 4, EPI_STORE>), dim3(N / 16), block, 0, stream, X, W, Y, M, N,
-                           K, 16, K);
+                           K, 16);
 }
 
 // out_float: 1 -> Y is float, 0 -> bfloat16.  Needs M <= 16, N % 16 == 0, K % 64 == 0.
@@ -147,28 +127,12 @@ SIA_EXPORT int sia_gemm_skinny(const void* X, const void* W, void* Y, int M, int
     return SIA_LAUNCH_CHECK();
 }
 
-// Partial sums: Y is float [splits][M][N] with splits = sia_gemm_skinny_splits(N, K) > 1.
-SIA_EXPORT int sia_gemm_skinny_partial(const void* X, const void* W, float* Y, int M, int N, int K, int splits,
-                                       hipStream_t stream) {
-    if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || N % 16 || K % 512 || splits < 1 || (K / 512) % splits) return SIA_BAD_ARGUMENT;
-    dim3 block(SK_WAVES * SIA_WAVE);
-    const int kps = K / splits;
-    if (N % 64 == 0 && N / 64 >= 256)
-        hipLaunchKernelGGL((gemm_skinny_kernel<float, 4, 1, EPI_PARTIAL>), dim3(N / 64, splits), block, 0, stream,
-                           (const bf16_t*)X, (const bf16_t*)W, Y, M, N, K, 16, kps);
-    else
-        hipLaunchKernelGGL((gemm_skinny_kernel<float, 1, 2, EPI_PARTIAL>), dim3(N / 16, splits), block, 0, stream,
-                           (const bf16_t*)X, (const bf16_t*)W, Y, M, N, K, 16, kps);
-    return SIA_LAUNCH_CHECK();
-}
-
 // Y[M, I] = silu(X Wg^T) * (X Wu^T) for W = [Wg; Wu] of 2 I rows.  Needs M <= 16, I % 16 == 0, K % 64 == 0.
 SIA_EXPORT int sia_gemm_skinny_swiglu(const void* X, const void* W, void* Y, int M, int inter, int K,
                                       hipStream_t stream) {
     if (M <= 0 || inter <= 0) return 0;
     if (M > 16 || inter % 16 || K % 64 || K <= 0) return SIA_BAD_ARGUMENT;
     hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 2, 2, EPI_SWIGLU>), dim3(inter / 16), dim3(SK_WAVES * SIA_WAVE), 0,
-                       stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, inter, K, inter, K);
+                       stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, inter, K, inter);
     return SIA_LAUNCH_CHECK();
 }
