@@ -26,12 +26,14 @@
 // probabilities are rounded to bfloat16 for the value product (reference:
 // kernels/attention_kernel.py:184-251 does the same in its prefill kernel).
 //
-// decode:  four waves per (split of the keys, kv head, sequence), each a contiguous quarter of the
-//          split; the query heads that share the kv head are the q columns (at most 16).  The four
-//          partial results are merged through LDS; (m, l, acc) per split go to a workspace and a
-//          second kernel combines the splits in order.
-// prefill: one wave per 16*NQ consecutive tokens of one query head; 4 waves a workgroup, which share
-//          each tile of keys and values through LDS (two stages; head sizes whose stages fit 64 KiB).
+// decode:  n_splits workgroups of four waves per (kv head, sequence); the sequence's tiles are dealt evenly, in
+//          order, to these waves (runs differ by a tile at most, whatever the length); the query heads that
+//          share the kv head are the q columns (at most 16).  A workgroup's four partial results are merged
+//          through LDS; (m, l, acc) per split go to a workspace and a second kernel combines the splits in
+//          order.
+// prefill: 128 consecutive tokens of one query head a workgroup (64 for head sizes over 128), as 4 waves of 32
+//          tokens or 8 waves of 16; the waves share each tile of keys and values through LDS (two stages;
+//          head sizes whose stages fit 64 KiB, the others load operands straight from the pages).
 #include "common.h"
 
 #ifndef SIA_HEAD_DIM

@@ -236,6 +236,24 @@ def test_matrix_core_attention_decode_and_mixed(hip, geom):
         torch.testing.assert_close(plain_kernel.float(), ref.float(), **tol(dtype))
 
 
+def test_matrix_core_attention_runs_longer_than_a_block_table_window(hip, monkeypatch):
+    """A wave holds 64 block-table entries at a time.  With pages of 64, runs of more than 4,096 keys that
+    start in the middle of a page (tiles are 32 keys) must reload the entries at a page's edge: one decoded
+    token over 17,500 keys (four runs of about 4,380 keys), and a prompt portion under a window of 5,000."""
+    n_heads, n_kv, D, ps = 2, 1, 16, 64
+    dtype = torch.bfloat16
+    monkeypatch.setattr(type(hip), "decode_split", staticmethod(lambda n_seqs, n_kv_heads, kv_bound: 1))
+    for q_lens, kv_lens, window in (([1], [17500], None), ([1], [17500], 9001), ([70], [9000], 5000)):
+        ctx = Ctx(q_lens, kv_lens)
+        cache = Cache(-(-kv_lens[0] // ps) + 3, n_kv, ps, D, dtype, kv_lens, seed=21)
+        cache.k_pages.copy_(rnd(*cache.k_pages.shape, dtype=dtype, seed=22))
+        cache.v_pages.copy_(rnd(*cache.v_pages.shape, dtype=dtype, seed=23))
+        qkv = rnd(ctx.n_tokens, (n_heads + 2 * n_kv) * D, dtype=dtype, seed=24, scale=3.0)
+        out = hip.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache)
+        ref = twin.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache)
+        torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("q_len", [1, 40])
 def test_attention_finds_one_key_at_every_kind_of_edge(hip, dtype, q_len):
