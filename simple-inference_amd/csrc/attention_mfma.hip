@@ -399,11 +399,15 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
 // ---------------------------------------------------------------------------------------------------
 // prefill: runs of several tokens (works for single tokens too, without splitting the keys)
 // ---------------------------------------------------------------------------------------------------
-// Two shapes of workgroup, both of PF_ROWS tokens: 4 waves of 32 tokens each (fewer reads from LDS per MFMA:
-// the faster one when there are workgroups enough to keep two on every compute unit), and 8 waves of 16
-// tokens each (two waves a SIMD from the start, so that one's softmax runs beside the other's MFMAs: the
-// faster one for short prompts and portions).  Head sizes above 128 take 4 waves of 16 tokens.
-constexpr int PF_ROWS = HD <= 128 ? 128 : 64;  // tokens per workgroup
+// Three shapes of workgroup.  Wide: 128 tokens, 4 waves of 32 tokens each, one tile of keys a step (fewest
+// instructions and reads from LDS per MFMA: the fastest when there are workgroups enough to keep two on every
+// compute unit).  Eight waves of 16 tokens: two waves a SIMD from the start, so that one's softmax runs beside
+// the other's MFMAs.  Split: 64 tokens, 8 waves: waves 0-3 take 16 tokens each and the even tiles of keys,
+// waves 4-7 the same tokens and the odd tiles, two tiles a step, and the two halves are merged through LDS at
+// the end: half as many steps for the last tokens of a prompt, whose many keys set the time of a short prompt
+// or portion.  Head sizes above 128 take 4 waves of 16 tokens.
+constexpr int PF_ROWS = HD <= 128 ? 128 : 64;  // tokens per wide workgroup
+constexpr int PF_ROWS_SPLIT = 64;              // tokens per split workgroup
 // Key and value tiles are shared by the workgroup's waves through LDS (two stages).  Rows are padded by
 // 16 bytes so that the 16 lanes of a 128-bit read hit 64 different banks.
 constexpr int K_STRIDE = HD + 8;                // elements per key row
@@ -507,13 +511,18 @@ __device__ __forceinline__ void compute_from_lds(const bf16_t* __restrict__ k_ld
     }
 }
 
-// PF_NQ groups of 16 tokens per wave, PF_WAVES waves: PF_NQ * PF_WAVES * 16 = PF_ROWS.
-template <int PF_NQ, int PF_WAVES>
+// PF_NQ groups of 16 tokens per wave; PF_WAVES waves, of which each KSPLIT-th part takes the same tokens and
+// every KSPLIT-th tile of keys: ROWS = PF_NQ * 16 * PF_WAVES / KSPLIT tokens per workgroup.
+template <int PF_NQ, int PF_WAVES, int KSPLIT>
 __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale,
     int window, int seq_begin, int seq_end) {
+    constexpr int ROW_WAVES = PF_WAVES / KSPLIT;
+    constexpr int ROWS = ROW_WAVES * PF_NQ * 16;
+    constexpr int TEAM = PF_WAVES * SIA_WAVE;
+    extern __shared__ __align__(16) unsigned char pf_lds[];
     // The chip has 8 dies (XCDs), each with an L2 of its own, and hands workgroups to them in turn.  The
     // workgroup ids are renumbered so that each die gets a contiguous range: the query heads that share a
     // kv head, and the row tiles of one head, then read their keys and values through one L2.
@@ -525,7 +534,7 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     // which sequence and which of its row tiles this workgroup has; late tiles (most keys) come first
     int tile = vid % gridDim.x, seq = seq_begin;
     for (; seq < seq_end; ++seq) {
-        const int tiles = (cu_q[seq + 1] - cu_q[seq] + PF_ROWS - 1) / PF_ROWS;
+        const int tiles = (cu_q[seq + 1] - cu_q[seq] + ROWS - 1) / ROWS;
         if (tile < tiles) {
             tile = tiles - 1 - tile;
             break;
@@ -535,9 +544,10 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     if (seq >= seq_end) return;
     const int hk = head / (n_heads / n_kv);
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    const int row_wave = wave % ROW_WAVES, part = wave / ROW_WAVES;  // which tokens, which tiles of a step
     const int q_begin = cu_q[seq], q_len = cu_q[seq + 1] - q_begin;
     const int first_pos = kv_len[seq] - q_len;
-    const int row0 = tile * PF_ROWS + wave * PF_NQ * 16;  // this wave's first row within the sequence's run
+    const int row0 = tile * ROWS + row_wave * PF_NQ * 16;  // this wave's first row within the sequence's run
     const bool wave_live = row0 < q_len;
     const int row_last = min(q_len - 1, row0 + PF_NQ * 16 - 1);
     const int* table = block_table + (size_t)seq * table_width;
@@ -561,52 +571,103 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     }
 
     if constexpr (PF_USE_LDS) {
-        __shared__ __align__(16) bf16_t k_lds[2][TILE * K_STRIDE];
-        __shared__ __align__(16) bf16_t v_lds[2][HD * V_STRIDE];
+        // LDS: [2 stages][KSPLIT tiles] of (keys, values)
+        constexpr int TILE_ELEMS = TILE * K_STRIDE + HD * V_STRIDE;
+        bf16_t* const lds_tiles = reinterpret_cast<bf16_t*>(pf_lds);
+#define PF_K_LDS(STAGE, PART) (lds_tiles + ((STAGE) * KSPLIT + (PART)) * TILE_ELEMS)
+#define PF_V_LDS(STAGE, PART) (PF_K_LDS(STAGE, PART) + TILE * K_STRIDE)
         // the workgroup's key range: from the first row's oldest visible key to the last live row's position
-        const int blk_rows = min(q_len - tile * PF_ROWS, PF_ROWS);
-        const int blk_hi = first_pos + tile * PF_ROWS + blk_rows - 1;
-        const int blk_lo = window > 0 ? max(0, first_pos + tile * PF_ROWS - window + 1) : 0;
+        const int blk_rows = min(q_len - tile * ROWS, ROWS);
+        const int blk_hi = first_pos + tile * ROWS + blk_rows - 1;
+        const int blk_lo = window > 0 ? max(0, first_pos + tile * ROWS - window + 1) : 0;
         const int wave_hi = first_pos + row_last;
         const int wave_lo = window > 0 ? max(0, first_pos + row0 - window + 1) : 0;
         const int kb_first = (blk_lo / TILE) * TILE, kb_last = (blk_hi / TILE) * TILE;
-        // Two register sets: while tile t is computed from LDS, tile t+1 waits in one set (its loads were
-        // issued an iteration ago) and the loads of tile t+2 are issued into the other.  The block-table
-        // window (64 entries from the page of the first tile it serves) is loaded outside the pipelined loop.
+        constexpr int STEP_KEYS = KSPLIT * TILE;
+        // Two register sets: while the tiles of step t are computed from LDS, those of step t+1 wait in one set
+        // (their loads were issued a step ago) and the loads of step t+2 are issued into the other.  The
+        // block-table window (64 entries from the page of the first tile it serves) is loaded outside the
+        // pipelined loop.
         for (int w_first = kb_first, w_end; w_first <= kb_last; w_first = w_end) {
             const int first_page = w_first >> ps_log2;
             w_end = (first_page + SIA_WAVE) << ps_log2;  // first key beyond the window, a multiple of TILE
             const int w_last = min(kb_last, w_end - TILE);
             PageWindow pages;
             pages_load(pages, table, table_width, first_page, lane);
-            TileRegs<PF_WAVES * SIA_WAVE> regs_a, regs_b;
-// One tile step: issue the loads of tile kb + 2 tiles into FREE, compute tile kb from LDS stage STAGE,
-// write the tile that waits in NEXT into the other stage.  (A macro, not a lambda: register sets that a
-// closure captures by reference end up in scratch memory.)
+            TileRegs<TEAM> regs_a[KSPLIT], regs_b[KSPLIT];
+// One step: issue the loads of the tiles two steps ahead into FREE, compute this wave's tile of the step at KB
+// from LDS stage STAGE, write the tiles that wait in NEXT into the other stage.  (Macros, not lambdas: register
+// sets that a closure captures by reference end up in scratch memory.)
+#define PF_FETCH(SET, KB)                                                                                       \
+    _Pragma("unroll") for (int p = 0; p < KSPLIT; ++p)                                                          \
+        tile_fetch(SET[p], kp, vp, pages, ps_log2, n_kv, hk, min((KB) + p * TILE, w_last), blk_lo, blk_hi)
+#define PF_STORE(SET, KB, STAGE)                                                                                \
+    _Pragma("unroll") for (int p = 0; p < KSPLIT; ++p)                                                          \
+        if ((KB) + p * TILE <= w_last) tile_store(SET[p], PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), ps_log2)
 #define PF_STEP(FREE, NEXT, KB, STAGE)                                                                          \
     do {                                                                                                        \
-        tile_fetch(FREE, kp, vp, pages, ps_log2, n_kv, hk, min((KB) + 2 * TILE, w_last), blk_lo, blk_hi);       \
-        if (wave_live && (KB) <= wave_hi && (KB) + TILE - 1 >= wave_lo)                                         \
-            compute_from_lds<PF_NQ>(k_lds[STAGE], v_lds[STAGE], qf, (KB), lo, hi, scale, m, l, acc);            \
-        if ((KB) + TILE <= w_last) tile_store(NEXT, k_lds[(STAGE) ^ 1], v_lds[(STAGE) ^ 1], ps_log2);           \
+        PF_FETCH(FREE, (KB) + 2 * STEP_KEYS);                                                                   \
+        const int my_kb = (KB) + part * TILE;                                                                   \
+        if (wave_live && my_kb <= w_last && my_kb <= wave_hi && my_kb + TILE - 1 >= wave_lo)                    \
+            compute_from_lds<PF_NQ>(PF_K_LDS(STAGE, part), PF_V_LDS(STAGE, part), qf, my_kb, lo, hi, scale, m,  \
+                                    l, acc);                                                                    \
+        PF_STORE(NEXT, (KB) + STEP_KEYS, (STAGE) ^ 1);                                                          \
         __syncthreads();                                                                                        \
     } while (0)
-            tile_fetch(regs_a, kp, vp, pages, ps_log2, n_kv, hk, w_first, blk_lo, blk_hi);
-            tile_fetch(regs_b, kp, vp, pages, ps_log2, n_kv, hk, min(w_first + TILE, w_last), blk_lo, blk_hi);
-            tile_store(regs_a, k_lds[0], v_lds[0], ps_log2);
+            PF_FETCH(regs_a, w_first);
+            PF_FETCH(regs_b, w_first + STEP_KEYS);
+            PF_STORE(regs_a, w_first, 0);
             __syncthreads();
-            for (int kb = w_first; kb <= w_last; kb += 2 * TILE) {
+            for (int kb = w_first; kb <= w_last; kb += 2 * STEP_KEYS) {
                 PF_STEP(regs_a, regs_b, kb, 0);
-                if (kb + TILE <= w_last) PF_STEP(regs_b, regs_a, kb + TILE, 1);
+                if (kb + STEP_KEYS <= w_last) PF_STEP(regs_b, regs_a, kb + STEP_KEYS, 1);
             }
 #undef PF_STEP
+#undef PF_STORE
+#undef PF_FETCH
         }
+#undef PF_K_LDS
+#undef PF_V_LDS
     } else {
+        static_assert(PF_USE_LDS || KSPLIT == 1, "the split shape stages its tiles through LDS");
         if (wave_live) {
             const int range_hi = first_pos + row_last;
             const int range_lo = window > 0 ? max(0, first_pos + row0 - window + 1) : 0;
             attend_range<PF_NQ>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, range_lo, range_hi, lo, hi, scale,
                                 m, l, acc);
+        }
+    }
+
+    if constexpr (KSPLIT == 2) {
+        // The waves of the second part hand (m, l, acc) to the waves of the first through LDS (the tiles are
+        // done with: the loop ended with a barrier), lane to lane, and those merge and write.
+        constexpr int PER_LANE = PF_NQ * (DBLOCKS * 4 + 2);
+        float* const box = reinterpret_cast<float*>(pf_lds) + (size_t)(row_wave * SIA_WAVE + lane) * PER_LANE;
+        if (part == 1) {
+#pragma unroll
+            for (int n = 0; n < PF_NQ; ++n) {
+                float* b = box + n * (DBLOCKS * 4 + 2);
+                b[0] = m[n];
+                b[1] = l[n];
+#pragma unroll
+                for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) b[2 + db * 4 + i] = acc[n][db][i];
+            }
+        }
+        __syncthreads();
+        if (part == 1) return;
+#pragma unroll
+        for (int n = 0; n < PF_NQ; ++n) {
+            const float* b = box + n * (DBLOCKS * 4 + 2);
+            const float m_other = b[0], m_new = fmaxf(m[n], m_other);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float w_mine = fast_exp2(m[n] - m_use), w_other = fast_exp2(m_other - m_use);
+            l[n] = l[n] * w_mine + b[1] * w_other;
+#pragma unroll
+            for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[n][db][i] = acc[n][db][i] * w_mine + b[2 + db * 4 + i] * w_other;
         }
     }
     if (!wave_live) return;
@@ -660,30 +721,55 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
     return SIA_LAUNCH_CHECK();
 }
 
-// Sequences seq_begin .. seq_end-1 of the step; n_tiles = sum over them of ceil(q_len / rows per workgroup).
+// Sequences seq_begin .. seq_end-1 of the step.  n_tiles = sum over them of ceil(q_len / sia_attn_prefill_rows()),
+// n_tiles_split the same with sia_attn_prefill_rows_split() (0 if this head size has no split shape).
 SIA_EXPORT int sia_attn_prefill_rows() { return PF_ROWS; }
+SIA_EXPORT int sia_attn_prefill_rows_split() { return (HD <= 128 && PF_USE_LDS) ? PF_ROWS_SPLIT : 0; }
+
+template <int NQ, int WAVES, int KSPLIT>
+static int launch_prefill(int tiles, const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
+                          const int* block_table, int table_width, const int* cu_q, const int* kv_len, void* out,
+                          int seq_begin, int seq_end, int n_heads, int n_kv, int ps_log2, float scale, int window,
+                          hipStream_t stream) {
+    constexpr int TILE_ELEMS = TILE * K_STRIDE + HD * V_STRIDE;
+    size_t lds_bytes = PF_USE_LDS ? (size_t)2 * KSPLIT * TILE_ELEMS * sizeof(bf16_t) : 0;
+    if (KSPLIT == 2) {
+        const size_t merge = (size_t)(WAVES / 2) * SIA_WAVE * NQ * (DBLOCKS * 4 + 2) * sizeof(float);
+        if (merge > lds_bytes) lds_bytes = merge;
+    }
+    const void* fn = reinterpret_cast<const void*>(&attn_prefill_kernel<NQ, WAVES, KSPLIT>);
+    if (lds_bytes > 48 * 1024) {  // beyond the default limit of dynamic LDS
+        const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL((attn_prefill_kernel<NQ, WAVES, KSPLIT>), dim3(tiles, n_heads), dim3(WAVES * SIA_WAVE),
+                       lds_bytes, stream, (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages,
+                       (const bf16_t*)v_pages, block_table, table_width, cu_q, kv_len, (bf16_t*)out, n_heads, n_kv,
+                       ps_log2, scale, window, seq_begin, seq_end);
+    return SIA_LAUNCH_CHECK();
+}
 
 SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                                 const int* block_table, int table_width, const int* cu_q, const int* kv_len,
-                                void* out, int seq_begin, int seq_end, int n_tiles, int n_heads, int n_kv,
-                                int page_size, float scale, int window, hipStream_t stream) {
+                                void* out, int seq_begin, int seq_end, int n_tiles, int n_tiles_split, int n_heads,
+                                int n_kv, int page_size, float scale, int window, hipStream_t stream) {
     if (seq_end <= seq_begin || n_tiles <= 0) return 0;
     const int ps_log2 = log2_exact(page_size);
     if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads > 65535 || q_row_stride % 8 || table_width <= 0)
         return SIA_BAD_ARGUMENT;
-#define LAUNCH(NQ, WAVES)                                                                                       \
-    hipLaunchKernelGGL((attn_prefill_kernel<NQ, WAVES>), dim3(n_tiles, n_heads), dim3(WAVES * SIA_WAVE), 0, stream,  \
-                       (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, \
-                       table_width, cu_q, kv_len, (bf16_t*)out, n_heads, n_kv, ps_log2, scale, window, seq_begin,  \
-                       seq_end)
+#define ARGS q, q_row_stride, k_pages, v_pages, block_table, table_width, cu_q, kv_len, out, seq_begin, seq_end, \
+             n_heads, n_kv, ps_log2, scale, window, stream
     if constexpr (HD > 128) {
-        LAUNCH(1, PF_ROWS / 16);
+        return launch_prefill<1, PF_ROWS / 16, 1>(n_tiles, ARGS);
     } else {
-        if ((long long)n_tiles * n_heads <= 2 * 256)  // not two workgroups for each of the 256 compute units
-            LAUNCH(1, PF_ROWS / 16);
-        else
-            LAUNCH(2, PF_ROWS / 32);
+        // Measured at 24 heads of 128 : the split shape is the fastest while all its
+        // workgroups are on the chip at once (prompts or portions up to about 1,024 tokens), the 8-wave shape
+        // of 128 tokens up to about 2,048, the wide shape beyond.
+        const long long wide_groups = (long long)n_tiles * n_heads;
+        if (PF_USE_LDS && n_tiles_split > 0 && wide_groups <= 224)
+            return launch_prefill<1, 2 * PF_ROWS_SPLIT / 16, 2>(n_tiles_split, ARGS);
+        if (wide_groups <= 480) return launch_prefill<1, PF_ROWS / 16, 1>(n_tiles, ARGS);
+        return launch_prefill<2, PF_ROWS / 32, 1>(n_tiles, ARGS);
     }
-#undef LAUNCH
-    return SIA_LAUNCH_CHECK();
+#undef ARGS
 }

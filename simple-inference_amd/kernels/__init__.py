@@ -46,8 +46,9 @@ _ATTN_SIGNATURES = {
     "sia_attn_decode": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                         _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_attn_prefill": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
-                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "sia_attn_prefill_rows": [],
+    "sia_attn_prefill_rows_split": [],
     "sia_attn_mfma_head_dim": [],
 }
 
@@ -324,12 +325,13 @@ class HipKernels:
                 n_kv_heads, cache.page_size, float(scale), window, n_splits, self._stream()),
                 "attn_decode")
         if n_dec < ctx.n_seqs:
-            rows = lib.sia_attn_prefill_rows()
+            rows, rows_split = lib.sia_attn_prefill_rows(), lib.sia_attn_prefill_rows_split()
             n_tiles = sum(-(-q // rows) for q in ctx.q_lens[n_dec:])
+            n_tiles_split = sum(-(-q // rows_split) for q in ctx.q_lens[n_dec:]) if rows_split else 0
             self._check(lib.sia_attn_prefill(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
-                _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_heads, n_kv_heads,
-                cache.page_size, float(scale), window, self._stream()), "attn_prefill")
+                _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_tiles_split, n_heads,
+                n_kv_heads, cache.page_size, float(scale), window, self._stream()), "attn_prefill")
 
     # -- sampling ------------------------------------------------------------------
     def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False):

@@ -236,6 +236,24 @@ def test_matrix_core_attention_decode_and_mixed(hip, geom):
         torch.testing.assert_close(plain_kernel.float(), ref.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("q_len, kv_len, window", [(130, 130, None), (900, 1000, None), (1900, 1900, None),
+                                                  (1900, 2100, 300)])
+def test_matrix_core_prefill_in_each_workgroup_shape(hip, q_len, kv_len, window):
+    """The prefill kernel picks one of three workgroup shapes by the number of workgroups: with 34 heads, 130
+    tokens take the split shape (64 tokens, even and odd key tiles on two sets of waves, merged at the end),
+    900 the 8-wave shape and 1,900 the wide one.  Lengths are no multiples of a tile."""
+    n_heads, n_kv, D, ps = 34, 2, 16, 16
+    dtype = torch.bfloat16
+    ctx = Ctx([q_len, 3], [kv_len, 40])
+    cache = Cache(-(-kv_len // ps) + 8, n_kv, ps, D, dtype, [kv_len, 40], seed=31)
+    cache.k_pages.copy_(rnd(*cache.k_pages.shape, dtype=dtype, seed=32))
+    cache.v_pages.copy_(rnd(*cache.v_pages.shape, dtype=dtype, seed=33))
+    qkv = rnd(ctx.n_tokens, (n_heads + 2 * n_kv) * D, dtype=dtype, seed=34, scale=2.0)
+    out = hip.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache)
+    ref = twin.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache)
+    torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
 def test_matrix_core_attention_runs_longer_than_a_block_table_window(hip, monkeypatch):
     """A wave holds 64 block-table entries at a time.  With pages of 64, runs of more than 4,096 keys that
     start in the middle of a page (tiles are 32 keys) must reload the entries at a page's edge: one decoded
