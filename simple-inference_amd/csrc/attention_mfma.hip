@@ -30,7 +30,7 @@
 //          order, to these waves (runs differ by a tile at most, whatever the length); the query heads that
 //          share the kv head are the q columns (at most 16).  A workgroup's four partial results are merged
 //          through LDS; (m, l, acc) per split go to a workspace and a second kernel combines the splits in
-//          order.
+//          order (a single split writes its result itself).
 // prefill: 128 consecutive tokens of one query head a workgroup (64 for head sizes over 128), as 4 waves of 32
 //          tokens or 8 waves of 16; the waves share each tile of keys and values through LDS (two stages;
 //          head sizes whose stages fit 64 KiB, the others load operands straight from the pages).
@@ -278,8 +278,8 @@ constexpr int DEC_WAVES = 4;
 __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
-    const int* __restrict__ kv_len, float* __restrict__ ws_acc, float* __restrict__ ws_ml, int n_heads, int n_kv,
-    int ps_log2, float scale, int window) {
+    const int* __restrict__ kv_len, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
+    bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window) {
     extern __shared__ float lds[];  // [DEC_WAVES][group][HD + 2]
     const int split = blockIdx.x, n_splits = gridDim.x, hk = blockIdx.y, seq = blockIdx.z;
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
@@ -337,6 +337,10 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
             const float wgt = fast_exp2(row[HD] - mx_use);  // a wave without keys has m = -inf: weight 0
             o += wgt * row[d];
             lsum += wgt * row[HD + 1];
+        }
+        if (n_splits == 1) {  // nothing to combine with: this is the result
+            out[((size_t)cu_q[seq] * n_heads + hk * group + c) * HD + d] = float_to_bf16(o * (1.f / lsum));
+            continue;
         }
         const size_t slot = ((size_t)seq * n_heads + hk * group + c) * n_splits + split;
         ws_acc[slot * HD + d] = o;
@@ -715,9 +719,11 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
     if (lds_bytes > 64 * 1024) return SIA_BAD_ARGUMENT;
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_splits, n_kv, n_seqs), dim3(DEC_WAVES * SIA_WAVE), lds_bytes,
                        stream, (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
-                       block_table, table_width, cu_q, kv_len, ws_acc, ws_ml, n_heads, n_kv, ps_log2, scale, window);
-    hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_heads, n_seqs), dim3(SIA_WAVE), 0, stream, ws_acc, ws_ml,
-                       cu_q, (bf16_t*)out, n_heads, n_splits);
+                       block_table, table_width, cu_q, kv_len, ws_acc, ws_ml, (bf16_t*)out, n_heads, n_kv, ps_log2,
+                       scale, window);
+    if (n_splits > 1)
+        hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_heads, n_seqs), dim3(SIA_WAVE), 0, stream, ws_acc,
+                           ws_ml, cu_q, (bf16_t*)out, n_heads, n_splits);
     return SIA_LAUNCH_CHECK();
 }
 
