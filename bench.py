@@ -139,17 +139,30 @@ def run_stream(preset_name, requests, max_running, max_seq_len, prefix_cache, ar
                                 generate_on_device=True)
     handles = [engine.add_request(p, params=SamplingParams(temperature=0.0, max_new_tokens=n, ignore_eos=True))
                for p, n in requests]
+    by_id = {h.id: h for h in handles}
+    first, last = {}, {}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     while engine.has_work():
-        engine.step()
+        emitted = engine.step()          # the tokens have reached the host when it returns
+        now = time.perf_counter() - t0
+        for rid in emitted:
+            first.setdefault(rid, now)
+            last[rid] = now
     torch.cuda.synchronize()
     sec = time.perf_counter() - t0
     assert all(len(h.generated) == n for h, (_, n) in zip(handles, requests))
     engine.cache.check()
+
+    def percentiles(values):
+        v = sorted(values)
+        return {f"p{q}": round(v[min(len(v) - 1, int(len(v) * q / 100))] * 1e3, 2) for q in (50, 90, 99)}
+    ttft = [first[i] for i in by_id]                       # every request is queued at time 0
+    tpot = [(last[i] - first[i]) / (len(by_id[i].generated) - 1) for i in by_id if len(by_id[i].generated) > 1]
     out = {"seconds": round(sec, 3), "steps": engine.stats["steps"], "prompt_tokens": sum(len(p) for p, _ in requests),
            "prefill_tokens_run": engine.stats["prefill_tokens"], "generated_tokens": engine.stats["decode_tokens"] + len(requests),
-           "generated_tok_s": round(sum(n for _, n in requests) / sec, 1)}
+           "generated_tok_s": round(sum(n for _, n in requests) / sec, 1),
+           "ttft_ms": percentiles(ttft), "tpot_ms": percentiles(tpot)}
     del engine
     torch.cuda.empty_cache()
     return out
