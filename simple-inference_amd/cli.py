@@ -53,7 +53,6 @@ def main(argv=None) -> int:
     import torch
 
     from . import Engine, EngineConfig, preset
-    from .config.registry import architecture_of
     from .weights import random_tensors, write_model_folder
 
     if args.write_model:

@@ -5,7 +5,6 @@ another layer's pages are registered, built and stepped without a change to the 
 They run on the CPU with the torch twins and on the GPU with the HIP kernels.
 """
 
-import copy
 
 import pytest
 import torch

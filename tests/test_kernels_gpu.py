@@ -50,7 +50,6 @@ class Ctx:
 
 class Cache:
     def __init__(self, n_pages, n_kv, page_size, head_dim, dtype, kv_lens, seed=0):
-        from types import SimpleNamespace
         self.page_size = page_size
         self.k_pages = torch.zeros(n_pages, n_kv, page_size, head_dim, dtype=dtype, device=DEV)
         self.v_pages = torch.zeros(n_pages, n_kv, head_dim, page_size, dtype=dtype, device=DEV)

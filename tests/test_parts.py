@@ -1,6 +1,5 @@
 """Each part alone against the plain implementation's function for it, at sizes of its own."""
 
-import math
 
 import pytest
 import torch
@@ -48,7 +47,6 @@ class OneSequence:
     """A step context and cache for one whole sequence of T tokens, made by the package's own runner pieces."""
 
     def __init__(self, env, T, need=None, page_size=8):
-        from simple_inference_amd.parts.plan import PagedKVNeed
         layout = CacheLayout()
         if need is not None:
             layout.kv_groups, layout.kv_slabs, layout.run_kv = [need], [1], [(0, 0)]

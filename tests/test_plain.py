@@ -8,7 +8,6 @@ by one) fails it.
 
 import math
 
-import pytest
 import torch
 import torch.nn.functional as F
 

@@ -7,7 +7,7 @@ import random
 import pytest
 import torch
 
-from helpers import TOLERANCE, Tiny, plain_logits, random_tokens, rel_err, write_tiny_model
+from helpers import TOLERANCE, Tiny, plain_logits, rel_err, write_tiny_model
 from test_trace_run import collect, make_trace
 
 pytestmark = pytest.mark.gpu

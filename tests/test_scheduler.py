@@ -1,7 +1,6 @@
 """The scheduler's decisions and the engine around it, on the CPU with the torch twins of the kernels."""
 
 import pytest
-import torch
 
 import plain_llama as plain
 from helpers import TINIES, random_tokens, write_tiny_model
