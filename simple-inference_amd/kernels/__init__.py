@@ -85,6 +85,9 @@ class HipKernels:
         self.core = build.load_library("core")
         _bind(self.core, _SIGNATURES)
         self._attn_libs = {}
+        # the short way to the current stream's handle, where this torch has it (a few microseconds less a launch)
+        self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        self._device_index = torch.device(device).index or 0
         self.use_mfma_attention = True   # tests switch it off to reach the plain kernel in bfloat16
         self.use_skinny_gemm = True      # few-row bfloat16 products by this package's kernel, not the library
         self._skinny_rows = self.core.sia_gemm_skinny_max_rows()
@@ -103,6 +106,9 @@ class HipKernels:
 
     # -- helpers -------------------------------------------------------------
     def _stream(self):
+        """Handle of torch's current stream on the device (during graph capture: the capturing stream)."""
+        if self._raw_stream is not None:
+            return self._raw_stream(self._device_index)
         return torch.cuda.current_stream(self.device).cuda_stream
 
     def _check(self, code: int, what: str):

@@ -23,6 +23,8 @@ class Sampler:
         rows = logits.shape[0]
         if rows != len(params) or rows != len(draw_indices):
             raise ValueError(f"{rows} logits rows, {len(params)} parameter sets, {len(draw_indices)} draw indices")
+        if all(p.greedy for p in params):    # nothing but the logits is needed: no parameter tensors, no copies
+            return self.kernels.sample(logits, None, None, None, None, all_greedy=True)
         host = torch.empty((4, rows), dtype=torch.float32)
         for i, (p, n) in enumerate(zip(params, draw_indices)):
             host[0, i] = p.temperature
@@ -30,5 +32,4 @@ class Sampler:
             host[2, i] = 0.0 if p.greedy else uniform_for(p.seed, n)
         top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32)
         dev = host.to(self.device)
-        return self.kernels.sample(logits, dev[0], top_k.to(self.device), dev[1], dev[2],
-                                   all_greedy=all(p.greedy for p in params))
+        return self.kernels.sample(logits, dev[0], top_k.to(self.device), dev[1], dev[2])

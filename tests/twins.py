@@ -115,6 +115,8 @@ class TwinKernels:
 
     # -- sampling --------------------------------------------------------------
     def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False):
+        if all_greedy:
+            return torch.argmax(logits.double(), dim=-1).to(torch.int32)
         out = []
         for r in range(logits.shape[0]):
             row = logits[r].double()
