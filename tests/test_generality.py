@@ -1,7 +1,8 @@
 """Parts that are not the served architecture's, defined here and plugged in from outside.
 
 A toy mixer with state of its own, a layer order that names a layer twice, and a mixer that reads
-another layer's pages are registered, built and stepped without a change to the package's files.
+another layer's pages are registered, built and stepped without a change to the package's files;
+so are a feed-forward that routes tokens to experts, a norm and a position encoding of other kinds.
 They run on the CPU with the torch twins and on the GPU with the HIP kernels.
 """
 
@@ -226,3 +227,152 @@ def test_each_run_of_a_layer_has_pages_of_its_own(toy_registered, backend):
         assert rel_err(got, want) <= (3e-2 if backend == "hip-bf16" else 2e-5)
     finally:
         unregister_architecture("ToyTwice")
+
+
+# ---- a feed-forward with routing, a norm and a position encoding of other kinds, from outside --------------------
+class TopOneExperts:
+    """Two small expert matrices and a router: every token goes through the expert its router score prefers,
+    weighted by the softmax of the two scores (float32 routing)."""
+
+    def __init__(self, params, env):
+        self.hidden, self.n = int(params["hidden_size"]), int(params["experts"])
+        self.env = env
+
+    def weight_specs(self):
+        specs = {"router": TensorSpec((self.n, self.hidden))}
+        for e in range(self.n):
+            specs[f"expert{e}"] = TensorSpec((self.hidden, self.hidden))
+        return specs
+
+    def bind(self, tensors):
+        self.router = tensors["router"]
+        self.experts = [tensors[f"expert{e}"] for e in range(self.n)]
+
+    def forward(self, h, ctx):
+        k = self.env.kernels
+        scores = k.linear(h, self.router, out_float32=True)
+        probs = torch.softmax(scores.float(), dim=-1)
+        choice = probs.argmax(dim=-1)
+        out = torch.zeros_like(h)
+        for e, w in enumerate(self.experts):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                y = k.linear(h[rows].contiguous(), w)
+                out[rows] = (y.float() * probs[rows, e:e + 1]).to(h.dtype)
+        return out
+
+
+class CenteredNorm:
+    """A norm that also takes the mean away (the package's takes none): same contract towards the stream."""
+
+    def __init__(self, params, env):
+        self.size, self.eps, self.env = int(params["size"]), float(params["eps"]), env
+
+    def weight_specs(self):
+        return {"weight": TensorSpec((self.size,), "vector")}
+
+    def bind(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, stream, rows=None):
+        if rows is None:
+            if stream.delta is not None:
+                stream.residual.add_(stream.delta.float())
+                stream.delta = None
+            x = stream.residual
+        else:
+            x = stream.residual[rows.long()]
+            if stream.delta is not None:
+                x = x + stream.delta[rows.long()].float()
+        x = x - x.mean(-1, keepdim=True)
+        return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight).to(self.env.dtype)
+
+
+class LinearAngles:
+    """Rotation angles that grow with the pair's index: angle(p, i) = p * step * (i + 1)."""
+
+    def __init__(self, params, env):
+        self.rotary_dim, self.step = int(params["rotary_dim"]), float(params["step"])
+        self.env = env
+
+    def weight_specs(self):
+        return {}
+
+    def bind(self, tensors):
+        pass
+
+    def tables(self):
+        pos = torch.arange(self.env.max_positions, dtype=torch.float32)
+        ang = torch.outer(pos, self.step * torch.arange(1, self.rotary_dim // 2 + 1, dtype=torch.float32))
+        return ang.cos().to(self.env.device).contiguous(), ang.sin().to(self.env.device).contiguous()
+
+
+def other_kinds_plan(cfg):
+    from simple_inference_amd.parts import PartSpec as P
+    norm = lambda name: P("test_centered", {"size": H, "eps": 1e-4}, {"weight": name})
+    pos = {"kind": "test_linear_angles", "params": {"rotary_dim": 16, "step": 0.05}}
+    layer = LayerSpec(
+        mixer=P("attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16, "position": pos},
+                {k: f"attn.{k}" for k in ("q", "k", "v", "o")}),
+        feed_forward=P("test_top_one", {"hidden_size": H, "experts": 2},
+                       {"router": "ffn.router", "expert0": "ffn.e0", "expert1": "ffn.e1"}),
+        mixer_norm=norm("n1"), feed_forward_norm=norm("n2"))
+    return ModelPlan(hidden_size=H, vocab_size=V,
+                     embedding=P("embedding", {"vocab_size": V, "hidden_size": H}, {"weight": "embed"}),
+                     layers=[layer], order=[0, 0], final_norm=norm("final"),
+                     head=P("head", {"vocab_size": V, "hidden_size": H, "tied": True}, {}))
+
+
+def other_kinds_reference(w, tokens):
+    import plain_llama as plain
+    w = {k: v.double() for k, v in w.items()}
+    T = len(tokens)
+    pos = torch.arange(T)
+    ang = torch.outer(pos.double(), 0.05 * torch.arange(1, 9).double())
+    cos, sin = torch.cat([ang.cos()] * 2, -1), torch.cat([ang.sin()] * 2, -1)
+
+    def norm(x, g):
+        x = x - x.mean(-1, keepdim=True)
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-4) * g
+
+    x = w["embed"][tokens]
+    for _ in range(2):
+        h = norm(x, w["n1"])
+        q = plain.apply_rope((h @ w["attn.q"].T).view(T, 2, 16), cos, sin)
+        k = plain.apply_rope((h @ w["attn.k"].T).view(T, 1, 16), cos, sin)
+        v = (h @ w["attn.v"].T).view(T, 1, 16)
+        x = x + plain.attention(q, k, v, pos, pos).reshape(T, 32) @ w["attn.o"].T
+        h = norm(x, w["n2"])
+        probs = torch.softmax(h @ w["ffn.router"].T, -1)
+        choice = probs.argmax(-1)
+        y = torch.stack([(h[t] @ w[f"ffn.e{int(choice[t])}"].T) * probs[t, choice[t]] for t in range(T)])
+        x = x + y
+    return norm(x, w["final"]) @ w["embed"].T
+
+
+@pytest.mark.parametrize("backend", [pytest.param("twins"), pytest.param("hip-f32", marks=pytest.mark.gpu)])
+def test_feed_forward_norm_and_position_encoding_of_other_kinds(backend):
+    from simple_inference_amd.parts import (
+        FEED_FORWARDS, NORMS, POSITION_ENCODINGS, register_feed_forward, register_norm, register_position_encoding,
+    )
+    register_feed_forward("test_top_one", TopOneExperts, replace=True)
+    register_norm("test_centered", CenteredNorm, replace=True)
+    register_position_encoding("test_linear_angles", LinearAngles, replace=True)
+    register_architecture("ToyOtherKinds", lambda d: d, other_kinds_plan, replace=True)
+    try:
+        runner, cache, weights = make(backend, {"architectures": ["ToyOtherKinds"]})
+        tokens = torch.randint(0, V, (23,), generator=torch.Generator().manual_seed(5)).tolist()
+        ref = other_kinds_reference(weights, tokens)
+        cache.admit(1)
+        got, fed = [], 0
+        for n in (9, 2, 1, 1, 7, 3):           # portions and single tokens, as for any architecture
+            got.append(runner.run([StepEntry(1, tokens[fed:fed + n], list(range(n)))]))
+            fed += n
+        assert rel_err(torch.cat(got), ref) < 3e-5
+        cache.release(1)
+        cache.check()
+    finally:
+        unregister_architecture("ToyOtherKinds")
+        FEED_FORWARDS.unregister("test_top_one")
+        NORMS.unregister("test_centered")
+        POSITION_ENCODINGS.unregister("test_linear_angles")
