@@ -48,6 +48,9 @@ def parse_args(argv=None):
     ap.add_argument("--points", default="1,64", help="further decode batch sizes to report, comma separated")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--temperature", type=float, default=0.0, help="sampling of the decode measurement (0: greedy)")
+    ap.add_argument("--top-k", type=int, default=0)
+    ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix"])
     ap.add_argument("--max-running", type=int, default=64, help="request slots of the stream workloads")
     return ap.parse_args(argv)
@@ -84,14 +87,16 @@ def random_prompt(vocab, n, seed):
     return torch.randint(0, vocab, (n,), generator=g).tolist()
 
 
-def measure_decode(engine, batch, context, steps, warmup, seed=0):
+def measure_decode(engine, batch, context, steps, warmup, seed=0, sampling=(0.0, 0, 1.0)):
     """(seconds per step, mean context over the timed steps) with ``batch`` requests decoding."""
     from simple_inference_amd import SamplingParams
 
     engine.reset()
     vocab = engine.model.vocab_size
-    params = SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + batch + 2, ignore_eos=True)
-    reqs = [engine.add_request(random_prompt(vocab, context, seed + i), params=params) for i in range(batch)]
+    temperature, top_k, top_p = sampling
+    reqs = [engine.add_request(random_prompt(vocab, context, seed + i), params=SamplingParams(
+        temperature=temperature, top_k=top_k, top_p=top_p, seed=seed + i, max_new_tokens=warmup + steps + batch + 2,
+        ignore_eos=True)) for i in range(batch)]
     while any(r.num_generated == 0 for r in reqs):   # prefill every prompt
         engine.step()
     for _ in range(warmup):
@@ -219,7 +224,8 @@ def main(argv=None):
     layer_w, head_w = matmul_params(mc)
 
     def decode_point(batch):
-        dt, ctx = measure_decode(engine, batch, args.context, args.steps, args.warmup, args.seed)
+        dt, ctx = measure_decode(engine, batch, args.context, args.steps, args.warmup, args.seed,
+                                 (args.temperature, args.top_k, args.top_p))
         bytes_read = (layer_w + head_w) * el + batch * ctx * mc.kv_bytes_per_token(el)
         return dt, batch / dt, bytes_read / dt / 1e9
 
@@ -236,6 +242,7 @@ def main(argv=None):
             "head_dim": mc.head_dim, "intermediate": mc.intermediate_size, "vocab": mc.vocab_size,
             "global_batch": args.batch, "seq_len": args.context, "context_limit": 4096,
             "page_size": engine.cfg.block_size, "graphs": engine.graphs is not None, "parallelism": "single GPU",
+            "sampling": "greedy" if args.temperature == 0 else f"T={args.temperature} k={args.top_k} p={args.top_p}",
         },
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(gbs / PEAK_HBM_GBS, 4)},

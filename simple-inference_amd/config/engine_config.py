@@ -44,7 +44,7 @@ class EngineConfig:
     chunk_tokens: int = 512               # most tokens one step runs (decoded tokens + prompt portions)
     dtype: str = "bfloat16"               # "bfloat16" (serving kernels) or "float32" (true 32-bit everywhere)
     eos_id: Optional[int] = None          # None → the model configuration's; -1 → never stop on a token
-    use_graphs: bool = False              # replay decode-only steps from captured hipGraphs
+    use_graphs: Optional[bool] = None     # replay decode-only steps from captured hipGraphs; None → on a GPU, yes
     use_prefix_cache: bool = False        # reuse complete pages of equal prompt prefixes
     prefix_cache_blocks: Optional[int] = None
     warmup: bool = False
@@ -66,6 +66,11 @@ class EngineConfig:
     @property
     def torch_dtype(self) -> torch.dtype:
         return resolve_dtype(self.dtype)
+
+    def graphs_wanted(self) -> bool:
+        if self.use_graphs is not None:
+            return bool(self.use_graphs)
+        return torch.device(self.device).type == "cuda"
 
     def pages_per_request(self) -> int:
         return -(-self.max_seq_len // self.block_size)

@@ -54,7 +54,7 @@ class Engine:
             cap = engine_cfg.prefix_cache_blocks or engine_cfg.resolved_num_kv_blocks()
             self.prefix_cache = PrefixCache(self.cache, max_pages=cap)
         self.graphs = None
-        if engine_cfg.use_graphs:
+        if engine_cfg.graphs_wanted():
             from .graphs import GraphedDecode
             self.graphs = GraphedDecode(self)
         self.stats = {"steps": 0, "tokens_run": 0, "prefill_tokens": 0, "decode_tokens": 0}

@@ -33,9 +33,8 @@ _SIGNATURES = {
     "sia_attention_generic": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
-    "sia_sample": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
-    "sia_argmax": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
-    "sia_argmax_workspace_per_row": [],
+    "sia_sample": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_sample_workspace_bytes": [_c_int],
     "sia_gemm_skinny": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_gemm_skinny_max_rows": [],
     "sia_gemm_skinny_swiglu": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -84,6 +83,7 @@ class HipKernels:
         self.device = torch.device(device)
         self.core = build.load_library("core")
         _bind(self.core, _SIGNATURES)
+        self.core.sia_sample_workspace_bytes.restype = ctypes.c_longlong
         self._attn_libs = {}
         # the short way to the current stream's handle, where this torch has it (a few microseconds less a launch)
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -340,24 +340,23 @@ class HipKernels:
                 n_kv_heads, cache.page_size, float(scale), window, self._stream()), "attn_prefill")
 
     # -- sampling ------------------------------------------------------------------
-    def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False):
-        """One token per row.  ``all_greedy`` (every temperature is 0, which the caller knows on the host)
-        takes the argmax kernels that spread a row over the chip."""
+    def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False, filters=None):
+        """One token per row.  What the caller knows on the host spares launches: ``all_greedy`` (every
+        temperature is 0; the parameter tensors may then be None), or ``filters``, the sum of 1 if some row
+        may have a top-k filter and 2 if some row may have a top-p filter below 1 (None: both)."""
         rows, vocab = logits.shape
         self._want(logits, "logits", torch.float32)
         if all_greedy:
-            out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-            per_row = self.core.sia_argmax_workspace_per_row()
-            ws_val = torch.empty((rows * per_row,), dtype=torch.float32, device=logits.device)
-            ws_idx = torch.empty((rows * per_row,), dtype=torch.int32, device=logits.device)
-            self._check(self.core.sia_argmax(_ptr(logits), _ptr(out), _ptr(ws_val), _ptr(ws_idx), rows, vocab,
-                                             self._stream()), "argmax")
-            return out
-        self._want(temperature, "temperature", torch.float32, (rows,))
-        self._want(top_k, "top_k", torch.int32, (rows,))
-        self._want(top_p, "top_p", torch.float32, (rows,))
-        self._want(uniform, "uniform", torch.float32, (rows,))
+            filters = 0
+            temperature = top_k = top_p = uniform = None
+        else:
+            filters = 4 | (3 if filters is None else int(filters) & 3)
+            self._want(temperature, "temperature", torch.float32, (rows,))
+            self._want(top_k, "top_k", torch.int32, (rows,))
+            self._want(top_p, "top_p", torch.float32, (rows,))
+            self._want(uniform, "uniform", torch.float32, (rows,))
         out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+        workspace = torch.zeros((self.core.sia_sample_workspace_bytes(rows),), dtype=torch.uint8, device=logits.device)
         self._check(self.core.sia_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
-                                         _ptr(out), rows, vocab, self._stream()), "sample")
+                                         _ptr(out), _ptr(workspace), rows, vocab, filters, self._stream()), "sample")
         return out

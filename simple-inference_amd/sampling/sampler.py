@@ -32,4 +32,5 @@ class Sampler:
             host[2, i] = 0.0 if p.greedy else uniform_for(p.seed, n)
         top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32)
         dev = host.to(self.device)
-        return self.kernels.sample(logits, dev[0], top_k.to(self.device), dev[1], dev[2])
+        filters = (1 if any(p.top_k > 0 for p in params) else 0) | (2 if any(0.0 < p.top_p < 1.0 for p in params) else 0)
+        return self.kernels.sample(logits, dev[0], top_k.to(self.device), dev[1], dev[2], filters=filters)

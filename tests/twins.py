@@ -114,7 +114,7 @@ class TwinKernels:
         return out.view(N, n_heads * head_dim).to(qkv.dtype)
 
     # -- sampling --------------------------------------------------------------
-    def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False):
+    def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False, filters=None):
         if all_greedy:
             return torch.argmax(logits.double(), dim=-1).to(torch.int32)
         out = []
