@@ -18,18 +18,18 @@
 //   3. top-p: the lowest kept value the same way, with the probability mass per digit in place of
 //      the count;
 //   4. the kept mass of each chunk, then one workgroup per row finds the chunk and the token.
-// Probabilities enter every sum as 40-bit fixed-point integers (exp(x - max) * 2^40, at most 2^57
-// for a row): integer sums do not depend on their order, so histograms can be built with atomics
-// and every workgroup that recomputes a sum gets the same bits.  A pass starts by recomputing, from
-// the histograms of the passes before it, what those passes decided; nothing but the histograms
-// travels between launches.  Launches whose filter no row asks for are skipped by the caller's hint.
+// Probabilities enter every sum as fixed-point integers (exp(x - max) * 2^s with the largest s that keeps
+// a row's sum below 2^63: 46 bits for 128,256 entries): integer sums do not depend on their order, so
+// histograms can be built with atomics and every workgroup that recomputes a sum gets the same bits.  A
+// token whose probability is below 2^-s of the most likely one's counts as zero.  A pass starts by
+// recomputing, from the histograms of the passes before it, what those passes decided; nothing but the
+// histograms travels between launches.  Launches whose filter no row asks for are skipped by the caller's hint.
 #include "common.h"
 
 #define SP_CHUNKS 16
 #define SP_THREADS 1024
 #define SP_PASSES 3
 #define SP_MAX_BINS 2048
-#define SP_FIXED_ONE 1099511627776.0f  // 2^40
 
 typedef unsigned long long u64;
 
@@ -50,7 +50,7 @@ __device__ __forceinline__ uint32_t ordered_key(float f) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-__device__ __forceinline__ u64 fixed_mass(float x, float mx) { return (u64)(expf(x - mx) * SP_FIXED_ONE); }
+__device__ __forceinline__ u64 fixed_mass(float x, float mx, float one) { return (u64)(expf(x - mx) * one); }
 
 __device__ __forceinline__ void take_better(float& bv, int& bi, float v, int i) {
     if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
@@ -120,7 +120,7 @@ __device__ __forceinline__ void refine_top_p(const u64* __restrict__ mass, int p
         above += mass[b];
     }
     const u64 owners = __ballot(digit >= 0);
-    if (!owners) return;  // no mass at all under these digits (cannot be: the row's maximum has mass 2^40)
+    if (!owners) return;  // no mass at all under these digits (cannot be: the row's maximum has the mass of one)
     const int src = __ffsll((long long)owners) - 1;  // the lowest lane with a kept bin holds the lowest kept bin
     digit = __shfl(digit, src, SIA_WAVE);
     above_digit = __shfl(above_digit, src, SIA_WAVE);
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_top_p_kernel(const float* _
                                                                   const float* __restrict__ temperature,
                                                                   const int* __restrict__ top_k,
                                                                   const float* __restrict__ top_p, int vocab,
-                                                                  SampleRow* __restrict__ ws, int pass) {
+                                                                  SampleRow* __restrict__ ws, int pass, float one) {
     __shared__ u64 hist[SP_MAX_BINS];
     const int chunk = blockIdx.x, r = blockIdx.y;
     const float T = temperature[r], p = top_p[r];
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_top_p_kernel(const float* _
         const float x = row[i] / T;
         const uint32_t key = ordered_key(x);
         if (key >= s.cut_k && (key & high_mask) == s.prefix_p) {
-            const u64 q = fixed_mass(x, s.mx);
+            const u64 q = fixed_mass(x, s.mx, one);
             if (q) atomicAdd(&hist[(key >> shift) & (bins - 1)], q);
         }
     }
@@ -268,7 +268,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kept_kernel(const float* __
                                                                  const float* __restrict__ temperature,
                                                                  const int* __restrict__ top_k,
                                                                  const float* __restrict__ top_p, int vocab,
-                                                                 SampleRow* __restrict__ ws) {
+                                                                 SampleRow* __restrict__ ws, float one) {
     __shared__ u64 sums[SP_THREADS / SIA_WAVE];
     const int chunk = blockIdx.x, r = blockIdx.y;
     const float T = temperature[r];
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kept_kernel(const float* __
     u64 sum = 0;
     for (int i = begin + threadIdx.x; i < end; i += SP_THREADS) {
         const float x = row[i] / T;
-        if (ordered_key(x) >= cut) sum += fixed_mass(x, s.mx);
+        if (ordered_key(x) >= cut) sum += fixed_mass(x, s.mx, one);
     }
     sum += lanes_above_sum(sum);  // lane 0 of each wave holds the wave's sum
     if (threadIdx.x % SIA_WAVE == 0) sums[threadIdx.x / SIA_WAVE] = sum;
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_pick_kernel(const float* __
                                                                  const float* __restrict__ top_p,
                                                                  const float* __restrict__ uniform,
                                                                  int* __restrict__ out, int vocab,
-                                                                 const SampleRow* __restrict__ ws) {
+                                                                 const SampleRow* __restrict__ ws, float one) {
     __shared__ u64 wave_sum[SP_THREADS / SIA_WAVE];
     __shared__ int picked;
     const int r = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid / SIA_WAVE;
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_pick_kernel(const float* __
     u64 mine = 0;
     for (int i = i0; i < i1; ++i) {
         const float x = row[i] / T;
-        if (ordered_key(x) >= cut) mine += fixed_mass(x, s.mx);
+        if (ordered_key(x) >= cut) mine += fixed_mass(x, s.mx, one);
     }
     // mass of the threads before this one
     u64 inc = mine;
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_pick_kernel(const float* __
         for (int i = i0; i < i1; ++i) {
             const float x = row[i] / T;
             if (ordered_key(x) >= cut) {
-                cum += fixed_mass(x, s.mx);
+                cum += fixed_mass(x, s.mx, one);
                 if (cum > target) { picked = i; break; }
             }
         }
@@ -386,6 +386,10 @@ SIA_EXPORT int sia_sample(const float* logits, const float* temperature, const i
     if (filters && (!temperature || !top_k || !top_p || !uniform)) return SIA_BAD_ARGUMENT;
     SampleRow* ws = (SampleRow*)workspace;
     const dim3 grid(SP_CHUNKS, rows), block(SP_THREADS);
+    int bits = 62;  // fixed point: vocab * 2^bits < 2^63
+    while (bits > 0 && ((long long)vocab << bits) >> bits != (long long)vocab) --bits;
+    while (bits > 0 && (double)vocab * (double)(1ull << bits) >= 9.2e18) --bits;
+    const float one = (float)(1ull << bits);
     hipLaunchKernelGGL(sample_max_kernel, grid, block, 0, stream, logits, vocab, ws);
     if (filters & 1)
         for (int pass = 0; pass < SP_PASSES; ++pass)
@@ -393,10 +397,11 @@ SIA_EXPORT int sia_sample(const float* logits, const float* temperature, const i
     if (filters & 2)
         for (int pass = 0; pass < SP_PASSES; ++pass)
             hipLaunchKernelGGL(sample_top_p_kernel, grid, block, 0, stream, logits, temperature, top_k, top_p, vocab,
-                               ws, pass);
+                               ws, pass, one);
     if (filters)
-        hipLaunchKernelGGL(sample_kept_kernel, grid, block, 0, stream, logits, temperature, top_k, top_p, vocab, ws);
+        hipLaunchKernelGGL(sample_kept_kernel, grid, block, 0, stream, logits, temperature, top_k, top_p, vocab, ws,
+                           one);
     hipLaunchKernelGGL(sample_pick_kernel, dim3(rows), block, 0, stream, logits, filters ? temperature : nullptr, top_k,
-                       top_p, uniform, out, vocab, ws);
+                       top_p, uniform, out, vocab, ws, one);
     return SIA_LAUNCH_CHECK();
 }

@@ -320,8 +320,51 @@ def test_sample_matches_twin(hip, vocab):
         assert got.tolist() == ref.tolist(), (seed, got.tolist(), ref.tolist())
 
 
+@pytest.mark.parametrize("vocab", [7, 331, 50257])
+def test_sample_filters_at_their_edges(hip, vocab):
+    """Rows made so that a filter's edge shows: equal values (kept or dropped together), a k that is one short
+    of everything, a p so small that only the top stays, a single dominant token, values of both signs far
+    apart, and draws at both ends of the unit interval.  The hints of which filters exist must not matter."""
+    g = torch.Generator().manual_seed(vocab)
+    rows = []
+    flat = torch.zeros(vocab)                                        # all equal
+    steps = torch.arange(vocab, dtype=torch.float32).flip(0) * 0.25   # strictly falling
+    pairs = (torch.arange(vocab) // 2).float().flip(0) * 0.5          # equal pairs
+    spike = torch.randn(vocab, generator=g); spike[vocab // 3] = 30.0
+    wide = torch.randn(vocab, generator=g) * 40.0
+    shuffled = steps[torch.randperm(vocab, generator=g)]
+    cases = []
+    for base in (flat, steps, pairs, spike, wide, shuffled):
+        ties = base is flat or base is pairs   # a sort splits equal values as it likes: no top-p oracle for them
+        for k, p in ((0, 1.0), (1, 1.0), (3, 1.0), (vocab - 1, 1.0), (0, 1e-6), (0, 0.5), (4, 0.7), (0, 0.999)):
+            if not (ties and p < 1.0):
+                cases.append((base, 0.8, k, p))
+    logits = torch.stack([c[0] for c in cases]).to(DEV)
+    temperature = torch.tensor([c[1] for c in cases], dtype=torch.float32, device=DEV)
+    top_k = torch.tensor([c[2] for c in cases], dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([c[3] for c in cases], dtype=torch.float32, device=DEV)
+    for u_value in (1e-6, 0.37, 0.999999):
+        u = torch.full((len(cases),), u_value, dtype=torch.float32, device=DEV)
+        got = hip.sample(logits, temperature, top_k, top_p, u)
+        ref = twin.sample(logits, temperature, top_k, top_p, u)
+        assert got.tolist() == ref.tolist(), (u_value, [i for i, (a, b) in enumerate(zip(got.tolist(), ref.tolist())) if a != b])
+    # equal values are kept or dropped together: under any top-p, all of a row of equal values can be drawn
+    n = 5
+    flat_rows = flat.repeat(n, 1).to(DEV)
+    u = torch.linspace(0.01, 0.99, n, device=DEV)
+    got = hip.sample(flat_rows, torch.full((n,), 0.8, device=DEV), torch.zeros(n, dtype=torch.int32, device=DEV),
+                     torch.full((n,), 0.3, device=DEV), u)
+    assert got.tolist() == [min(vocab - 1, int(x * vocab)) for x in u.tolist()]
+    # rows without a filter, sampled with the hint that there is none
+    plain_rows = [i for i, c in enumerate(cases) if c[2] == 0 and c[3] == 1.0]
+    sel = torch.tensor(plain_rows, device=DEV)
+    u = torch.full((len(plain_rows),), 0.61, dtype=torch.float32, device=DEV)
+    args = (logits[sel].contiguous(), temperature[sel].contiguous(), top_k[sel].contiguous(), top_p[sel].contiguous(), u)
+    assert hip.sample(*args, filters=0).tolist() == hip.sample(*args).tolist() == twin.sample(*args).tolist()
+
+
 @pytest.mark.parametrize("vocab", [5, 1001, 4096, 128256])
-def test_argmax_over_the_chip_matches_the_one_workgroup_argmax(hip, vocab):
+def test_argmax_of_all_greedy_steps(hip, vocab):
     rows = 9
     logits = rnd(rows, vocab, seed=3, scale=3.0)
     logits[1] = 0.0                                   # all equal: index 0
