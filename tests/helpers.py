@@ -10,8 +10,9 @@ import torch
 
 import plain_llama as plain
 
-# Three tiny configurations that differ in every size and option.  A and B are the two of
-# BASELINE.json; C has sizes that are no power of two, a head size that is not
+# Three tiny configurations that differ in every size and option.  A: 2 layers, 4 query / 2 key-value
+# heads of 16, tied head, no frequency scaling, pages of 4.  B: 3 layers, 3 / 1 heads of 32, untied head,
+# llama3 scaling, pages of 8.  C has sizes that are no power of two, a head size that is not
 # hidden / heads, as many key/value heads as query heads, and another scaling.
 TINY_A = {
     "architectures": ["LlamaForCausalLM"], "model_type": "llama",
