@@ -19,6 +19,7 @@ torch's current stream, so they are captured with the library products between t
 
 from __future__ import annotations
 
+import gc
 from typing import Dict, List
 
 import numpy as np
@@ -64,7 +65,8 @@ class _Bucket:
 
 class GraphedDecode:
     def __init__(self, engine):
-        self.engine = engine
+        # no reference to the engine itself is kept: engine and graphs would form a cycle, and graphs that
+        # only the cycle collector frees may be destroyed while another engine is capturing, which HIP refuses
         self.runner = engine.runner
         self.cache = engine.cache
         self.device = engine.device
@@ -147,8 +149,14 @@ class GraphedDecode:
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            b.logits = model.forward(b.ctx, b.caches)
+        collecting = gc.isenabled()
+        gc.disable()   # no destructor of an older graph may run while the stream is capturing
+        try:
+            with torch.cuda.graph(graph):
+                b.logits = model.forward(b.ctx, b.caches)
+        finally:
+            if collecting:
+                gc.enable()
         b.graph = graph
         self._made[(size, kv_bound)] = b
         return b

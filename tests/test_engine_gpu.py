@@ -106,3 +106,43 @@ def test_temperature_sampling_on_the_gpu_follows_the_request_seed(folders):
             logits = plain.forward(cfg, w, toks)[-1]
             assert t == plain.sample_with_uniform(logits, uniform_for(sp.seed, n), sp.temperature, sp.top_k, sp.top_p)
             toks.append(t)
+
+
+@pytest.mark.parametrize("name", ["b", "c"])
+def test_random_request_streams_generate_what_each_request_generates_alone(folders, name):
+    """Forty requests of random lengths, with and without shared prefixes, greedy and sampled with seeds of their
+    own, arrive a few per step and run through engines with few pages, small portions, graphs and prefix reuse:
+    every request generates exactly the tokens it generates when it runs alone (32-bit, so that no rounding
+    difference between batch shapes can flip a token).  Several engines with graphs are made and dropped in turn."""
+    import random
+    folder, tiny = folders[name], TINIES[name]
+    V = tiny.config["vocab_size"]
+    rng = random.Random(7)
+    shared = [rng.randrange(V) for _ in range(60)]
+    reqs = []
+    for _ in range(40):
+        base = shared[:rng.randint(0, len(shared))] if rng.random() < 0.5 else []
+        prompt = base + [rng.randrange(V) for _ in range(rng.randint(1, 120))]
+        params = SamplingParams(temperature=rng.choice([0.0, 0.0, 0.7, 1.5]), top_k=rng.choice([0, 5, 40]),
+                                top_p=rng.choice([1.0, 0.9, 0.5]), seed=rng.randrange(1 << 30),
+                                max_new_tokens=rng.randint(1, 40), ignore_eos=True)
+        reqs.append((prompt, params))
+
+    def run(requests, stagger, **kw):
+        eng = Engine.from_folder(folder, EngineConfig(dtype="float32", max_seq_len=320, block_size=16, eos_id=-1, **kw))
+        handles, pending, step = [], list(requests), 0
+        while pending or eng.has_work():
+            for _ in range(min(len(pending), random.Random(step).randint(0, 3) if stagger else len(pending))):
+                prompt, params = pending.pop(0)
+                handles.append(eng.add_request(prompt, params=params))
+            eng.step()
+            step += 1
+        eng.cache.check()
+        return [h.generated for h in handles]
+
+    alone = [run([r], False, max_running=1, num_kv_blocks=64, use_graphs=False)[0] for r in reqs]
+    for kw in (dict(max_running=6, num_kv_blocks=60, chunk_tokens=32, use_graphs=True, use_prefix_cache=True),
+               dict(max_running=4, num_kv_blocks=40, chunk_tokens=16, use_graphs=True),
+               dict(max_running=16, num_kv_blocks=400, chunk_tokens=512, use_graphs=False, use_prefix_cache=True)):
+        got = run(reqs, True, **kw)
+        assert [i for i, (a, b) in enumerate(zip(got, alone)) if a != b] == [], kw
