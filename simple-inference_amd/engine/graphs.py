@@ -51,11 +51,13 @@ def kv_buckets_for(max_seq_len: int, smallest: int = 512) -> List[int]:
 
 
 class _Bucket:
-    def __init__(self, size, kv_bound, meta, host, offsets, ctx, caches):
+    def __init__(self, size, kv_bound, meta, host, offsets, ctx, caches, pinned):
         self.size = size
         self.kv_bound = kv_bound
         self.meta = meta          # device int32 buffer, fixed address
-        self.host = host          # host mirror that is filled and copied over
+        self.host = host          # host mirror that is filled and copied over (a numpy view of `pinned`)
+        self.pinned = pinned
+        self.copied = None        # event after the last copy of the mirror to the device
         self.offsets = offsets
         self.ctx = ctx
         self.caches = caches
@@ -96,7 +98,9 @@ class GraphedDecode:
         offsets = [0]
         for s in sizes:
             offsets.append(offsets[-1] + s)
-        host = np.zeros(offsets[-1], dtype=np.int32)
+        # the host mirror is pinned, so that the copy to the device needs no staging and does not wait
+        pinned = torch.zeros(offsets[-1], dtype=torch.int32, pin_memory=True)
+        host = pinned.numpy()
         meta = torch.zeros(offsets[-1], dtype=torch.int32, device=self.device)
         part = lambda i: meta[offsets[i]:offsets[i + 1]]
         ctx = StepContext(
@@ -106,12 +110,14 @@ class GraphedDecode:
             n_decode_seqs=size, q_lens=[1] * size, kv_bound=kv_bound)
         ctx.block_tables = [part(7 + g).view(size, self.width) for g in range(n_groups)]
         caches = self.cache.layer_caches(ctx.block_tables)
-        return _Bucket(size, kv_bound, meta, host, offsets, ctx, caches)
+        return _Bucket(size, kv_bound, meta, host, offsets, ctx, caches, pinned)
 
     def _fill(self, b: _Bucket, entries: List[StepEntry]) -> None:
         """Takes this step's pages and writes the step's metadata (padding included) into the buffers."""
         size, off, host = b.size, b.offsets, b.host
         cache = self.cache
+        if b.copied is not None:
+            b.copied.synchronize()   # the last copy has read the mirror (long done, unless nobody read that step's result)
         tok, pos, sot, cu, kvl, slots, rows = (host[off[i]:off[i + 1]] for i in range(7))
         tok[:] = 0
         pos[:] = 0
@@ -133,7 +139,10 @@ class GraphedDecode:
                 base = off[7 + g] + s * self.width
                 host[base:base + len(row)] = row
                 host[base + len(row):base + self.width] = -1
-        b.meta.copy_(torch.from_numpy(host))
+        b.meta.copy_(b.pinned, non_blocking=True)
+        if b.copied is None:
+            b.copied = torch.cuda.Event()
+        b.copied.record()
 
     # -- capture and replay -----------------------------------------------------------
     @torch.no_grad()
