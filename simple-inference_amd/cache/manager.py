@@ -55,6 +55,7 @@ class PagedGroup:
         self.scratch_page = num_pages
         self.allocator = PageAllocator(num_pages)
         self.tables: Dict[int, List[int]] = {}
+        self.versions: Dict[int, int] = {}   # bumped whenever a request's table changes (graph replay skips rows that did not)
         self.k = self.v = None
         if allocate_storage:
             shape_k = (slabs, num_pages + 1, need.num_kv_heads, page_size, need.head_dim)
@@ -75,6 +76,7 @@ class PagedGroup:
     def begin(self, req: int, reserve: int) -> None:
         self.allocator.reserve(req, reserve)
         self.tables[req] = []
+        self.versions[req] = 0
 
     def extend(self, req: int, start: int, end: int) -> None:
         """Makes the table ready for a step that writes positions ``start .. end-1``."""
@@ -85,12 +87,15 @@ class PagedGroup:
                 if table[idx] >= 0:
                     self.allocator.free_page(req, table[idx], back_to_reservation=True)
                     table[idx] = -1
+                    self.versions[req] += 1
         while len(table) < pages_for(end, self.page_size):
             table.append(self.allocator.allocate(req))
+            self.versions[req] += 1
 
     def release(self, req: int) -> None:
         self.allocator.release(req)
         self.tables.pop(req, None)
+        self.versions.pop(req, None)
 
 
 class StateSlots:
@@ -177,6 +182,7 @@ class CacheManager:
             for page in shared:
                 g.allocator.share(req, page)
                 g.tables[req].append(page)
+                g.versions[req] += 1
         self.lengths[req] = len(shared) * self.page_size
         return slot
 

@@ -58,6 +58,7 @@ class _Bucket:
         self.host = host          # host mirror that is filled and copied over (a numpy view of `pinned`)
         self.pinned = pinned
         self.copied = None        # event after the last copy of the mirror to the device
+        self.rows = {}            # (group, row) -> what the mirror's block-table row holds: (request, table version) or "pad"
         self.offsets = offsets
         self.ctx = ctx
         self.caches = caches
@@ -126,19 +127,27 @@ class GraphedDecode:
         sot[:] = np.arange(size)
         cu[:] = np.arange(size + 1)
         rows[:] = np.arange(size)
-        for g, grp in enumerate(cache.groups):
-            host[off[7 + g]:off[8 + g]] = grp.scratch_page
         for s, e in enumerate(entries):
             start = cache.extend(e.req, 1)
             tok[s] = e.tokens[0]
             pos[s] = start
             kvl[s] = start + 1
             slots[s] = cache.slot(e.req)
-            for g in range(len(cache.groups)):
-                row = cache.table(g, e.req)
+        # block tables: a row is rewritten only if it held another request or the request's table has changed
+        for g, grp in enumerate(cache.groups):
+            for s in range(size):
                 base = off[7 + g] + s * self.width
-                host[base:base + len(row)] = row
-                host[base + len(row):base + self.width] = -1
+                if s < len(entries):
+                    req = entries[s].req
+                    holds = (req, grp.versions[req])
+                    if b.rows.get((g, s)) != holds:
+                        row = grp.tables[req]
+                        host[base:base + len(row)] = row
+                        host[base + len(row):base + self.width] = -1
+                        b.rows[(g, s)] = holds
+                elif b.rows.get((g, s)) != "pad":
+                    host[base:base + self.width] = grp.scratch_page
+                    b.rows[(g, s)] = "pad"
         b.meta.copy_(b.pinned, non_blocking=True)
         if b.copied is None:
             b.copied = torch.cuda.Event()
