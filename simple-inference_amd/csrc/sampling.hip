@@ -374,7 +374,8 @@ __global__ __launch_bounds__(SP_THREADS) void sample_pick_kernel(const float* __
 
 SIA_EXPORT long long sia_sample_workspace_bytes(int rows) { return (long long)rows * (long long)sizeof(SampleRow); }
 
-// One token per row.  workspace: sia_sample_workspace_bytes(rows) bytes, all zero.  filters: bit 0 set if
+// One token per row.  workspace: sia_sample_workspace_bytes(rows) bytes, all zero (with filters == 0 they may
+// hold anything).  filters: bit 0 set if
 // some row may have a top-k filter, bit 1 if some row may have a top-p filter in (0, 1), bit 2 if some row has
 // a temperature above 0; launches for filters that no row has are skipped (rows decide for themselves inside
 // the launches that run).  With filters == 0 the parameter pointers may be null: every row takes its argmax.

@@ -120,19 +120,20 @@ class GraphedDecode:
         if b.copied is not None:
             b.copied.synchronize()   # the last copy has read the mirror (long done, unless nobody read that step's result)
         tok, pos, sot, cu, kvl, slots, rows = (host[off[i]:off[i + 1]] for i in range(7))
-        tok[:] = 0
-        pos[:] = 0
-        kvl[:] = 1
-        slots[:] = cache.slots.scratch_slot
-        sot[:] = np.arange(size)
-        cu[:] = np.arange(size + 1)
-        rows[:] = np.arange(size)
-        for s, e in enumerate(entries):
-            start = cache.extend(e.req, 1)
-            tok[s] = e.tokens[0]
-            pos[s] = start
-            kvl[s] = start + 1
-            slots[s] = cache.slot(e.req)
+        if not b.rows:   # first fill: what never changes
+            sot[:] = np.arange(size)
+            cu[:] = np.arange(size + 1)
+            rows[:] = np.arange(size)
+        n = len(entries)
+        starts = [cache.extend(e.req, 1) for e in entries]
+        tok[:n] = [e.tokens[0] for e in entries]
+        pos[:n] = starts
+        kvl[:n] = pos[:n] + 1
+        slots[:n] = [cache.slot(e.req) for e in entries]
+        tok[n:] = 0           # padding rows: token 0 at position 0 of the scratch page and slot
+        pos[n:] = 0
+        kvl[n:] = 1
+        slots[n:] = cache.slots.scratch_slot
         # block tables: a row is rewritten only if it held another request or the request's table has changed
         for g, grp in enumerate(cache.groups):
             for s in range(size):

@@ -356,7 +356,9 @@ class HipKernels:
             self._want(top_p, "top_p", torch.float32, (rows,))
             self._want(uniform, "uniform", torch.float32, (rows,))
         out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-        workspace = torch.zeros((self.core.sia_sample_workspace_bytes(rows),), dtype=torch.uint8, device=logits.device)
+        # the histograms of the filters start at zero; an argmax-only call reads nothing that it has not written
+        make = torch.zeros if filters else torch.empty
+        workspace = make((self.core.sia_sample_workspace_bytes(rows),), dtype=torch.uint8, device=logits.device)
         self._check(self.core.sia_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
                                          _ptr(out), _ptr(workspace), rows, vocab, filters, self._stream()), "sample")
         return out
