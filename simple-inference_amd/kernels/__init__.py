@@ -38,6 +38,8 @@ _SIGNATURES = {
     "sia_gemm_skinny": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_gemm_skinny_max_rows": [],
     "sia_gemm_skinny_swiglu": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_gemm_skinny_rope": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                             _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
 }
 
 
@@ -268,6 +270,39 @@ class HipKernels:
             _ptr(ctx.positions), _ptr(ctx.seq_of_token), _ptr(table), table_w, _ptr(k_pages), _ptr(v_pages),
             n, n_heads, n_kv_written, head_dim, rotary_dim, page_size, _DT[qkv.dtype], self._stream()),
             "rope_kv_write")
+
+    def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache):
+        """The q/k/v product, the rotation of q and k and the write of k and v into the pages.  Returns the
+        ``[tokens, (n_heads + 2 n_kv_written) head_dim]`` matrix whose q columns hold the rotated queries; its
+        k and v columns are not to be read (for few rows one kernel does all three and never writes them)."""
+        M, K = x.shape
+        if (self.use_skinny_gemm and n_kv_written and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
+                and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 32 == 0 and K % 64 == 0
+                and not ((n_heads + 2 * n_kv_written) * head_dim < 4096 and K > 4096)):
+            self._want(x, "q/k/v input")
+            self._want(w_qkv, "q/k/v weight")
+            width = (n_heads + 2 * n_kv_written) * head_dim
+            if tuple(w_qkv.shape) != (width, K):
+                raise KernelError(f"q/k/v weight {tuple(w_qkv.shape)} is not [{width}, {K}]")
+            if M != ctx.n_tokens:
+                raise KernelError(f"q/k/v input has {M} rows, the step {ctx.n_tokens} tokens")
+            for t, what in ((cos, "cos table"), (sin, "sin table")):
+                self._want(t, what, torch.float32)
+                if t.shape[1] != rotary_dim // 2 or t.shape[0] <= ctx.max_kv_len - 1:
+                    raise KernelError(f"{what} {tuple(t.shape)} does not cover position {ctx.max_kv_len - 1} "
+                                      f"with {rotary_dim // 2} pairs")
+            self._check_pages(cache.k_pages, cache.v_pages, cache.block_table, cache.page_size, n_kv_written,
+                              head_dim, x.dtype, ctx)
+            qkv = torch.empty((M, width), dtype=torch.bfloat16, device=x.device)
+            self._check(self.core.sia_gemm_skinny_rope(
+                _ptr(x), _ptr(w_qkv), _ptr(qkv), M, K, _ptr(cos), _ptr(sin), _ptr(ctx.positions),
+                _ptr(ctx.seq_of_token), _ptr(cache.block_table), cache.block_table.shape[1], _ptr(cache.k_pages),
+                _ptr(cache.v_pages), n_heads, n_kv_written, head_dim, cache.page_size, self._stream()),
+                "gemm_skinny_rope")
+            return qkv
+        qkv = self.linear(x, w_qkv)
+        self.rope_kv_write(qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache)
+        return qkv
 
     def _check_pages(self, k_pages, v_pages, table, page_size, n_kv, head_dim, dtype, ctx):
         self._want(k_pages, "key pages", dtype)

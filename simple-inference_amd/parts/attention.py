@@ -86,10 +86,9 @@ class Attention:
 
     def forward(self, h, ctx, cache):
         k = self.env.kernels
-        qkv = k.linear(h, self.w_qkv)
         cos, sin = self.position.tables()
-        k.rope_kv_write(
-            qkv, self.num_heads, self.num_kv_heads if self.writes_kv else 0, self.head_dim,
+        qkv = k.qkv_to_cache(
+            h, self.w_qkv, self.num_heads, self.num_kv_heads if self.writes_kv else 0, self.head_dim,
             self.position.rotary_dim, cos, sin, ctx, cache)
         out = k.paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, ctx, cache)

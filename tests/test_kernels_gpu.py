@@ -118,7 +118,7 @@ def test_gemm_generic(hip, dtype, shape):
     if dtype == torch.bfloat16:
         out = hip.gemm_generic(x, w)
         assert out.dtype == torch.bfloat16
-        torch.testing.assert_close(out.double(), ref, rtol=1e-2, atol=1e-2)
+        torch.testing.assert_close(out.double(), ref, **tol(dtype))
 
 
 @pytest.mark.parametrize("shape", [(1, 48, 64), (8, 5120, 3072), (16, 3072, 8192), (3, 16, 320), (11, 1008, 1024)])
@@ -205,6 +205,62 @@ def test_rope_kv_write_and_attention(hip, dtype, geom):
         out = hip.paged_attention(q2, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, c_twin)
         ref = twin.paged_attention(q2, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, c_twin)
         torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("geom", [
+    # heads, kv heads, head_dim, page_size, hidden, rows
+    (24, 8, 128, 64, 3072, 8), (3, 1, 32, 8, 192, 16), (5, 5, 96, 16, 1088, 1), (2, 1, 256, 32, 64, 5),
+    (7, 7, 64, 4, 2048, 13),
+])
+def test_qkv_product_that_rotates_and_writes_the_pages(hip, geom):
+    """Few rows: one kernel multiplies, rotates q and k and writes k and v into the pages.  Compared with the
+    product, rotation and write done one after the other on float sums (the twin rounds the product first, so
+    its result is a rounding away)."""
+    n_heads, n_kv, D, ps, hidden, rows = geom
+    dtype = torch.bfloat16
+    kv_lens = [3 + 41 * i for i in range(rows)]
+    kv_lens[-1] = 2 * ps  # a token in the last slot of a page
+    if rows > 1:
+        kv_lens[0] = ps + 1  # and one in the first
+    ctx = Ctx([1] * rows, kv_lens)
+    pages = sum(-(-kv // ps) for kv in kv_lens) + 3
+    c_hip = Cache(pages, n_kv, ps, D, dtype, kv_lens, seed=4)
+    c_ref = Cache(pages, n_kv, ps, D, torch.float32, kv_lens, seed=4)  # float pages: rounded once, at the comparison
+    c_hip.k_pages.copy_(rnd(*c_hip.k_pages.shape, dtype=dtype, seed=5)); c_ref.k_pages.copy_(c_hip.k_pages)
+    c_hip.v_pages.copy_(rnd(*c_hip.v_pages.shape, dtype=dtype, seed=6)); c_ref.v_pages.copy_(c_hip.v_pages)
+    x = rnd(rows, hidden, dtype=dtype, seed=7)
+    w = rnd((n_heads + 2 * n_kv) * D, hidden, dtype=dtype, seed=8, scale=hidden ** -0.5)
+    pos = torch.arange(max(kv_lens) + 1, dtype=torch.float32)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    ang = torch.outer(pos, inv)
+    cos, sin = ang.cos().to(DEV), ang.sin().to(DEV)
+    launched = []
+    real = hip.core.sia_gemm_skinny_rope
+    hip.core.sia_gemm_skinny_rope = lambda *a: launched.append(1) or real(*a)
+    try:
+        qkv = hip.qkv_to_cache(x, w, n_heads, n_kv, D, D, cos, sin, ctx, c_hip)
+    finally:
+        hip.core.sia_gemm_skinny_rope = real
+    assert launched, "the fused kernel did not run"
+    # reference: float product, rotated in float, rounded once
+    ref = (x.float() @ w.float().T)
+    twin.rope_kv_write(ref, n_heads, n_kv, D, D, cos, sin, ctx, c_ref)
+    nq = n_heads * D
+    torch.testing.assert_close(qkv[:, :nq].float(), ref[:, :nq], **tol(dtype))
+    torch.testing.assert_close(c_hip.k_pages.float(), c_ref.k_pages, **tol(dtype))
+    torch.testing.assert_close(c_hip.v_pages.float(), c_ref.v_pages, **tol(dtype))
+    # nothing but the tokens' own slots has changed
+    before = rnd(*c_hip.k_pages.shape, dtype=dtype, seed=5)
+    changed = (c_hip.k_pages != before).any(dim=-1)            # [page, kv head, offset]
+    assert int(changed.any(dim=1).sum()) <= rows
+    # and the separate path gives the same within the rounding of the product
+    qkv2 = hip.linear(x, w)
+    c_two = Cache(pages, n_kv, ps, D, dtype, kv_lens, seed=4)
+    c_two.k_pages.copy_(before); c_two.v_pages.copy_(rnd(*c_hip.v_pages.shape, dtype=dtype, seed=6))
+    hip.rope_kv_write(qkv2, n_heads, n_kv, D, D, cos, sin, ctx, c_two)
+    torch.testing.assert_close(qkv[:, :nq].float(), qkv2[:, :nq].float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(c_hip.k_pages.float(), c_two.k_pages.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(c_hip.v_pages.float(), c_two.v_pages.float(), rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("geom", [

@@ -49,6 +49,11 @@ class TwinKernels:
         g, u = gu[:, :inter].float(), gu[:, inter:].float()
         return (g * torch.sigmoid(g) * u).to(gu.dtype)
 
+    def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache):
+        qkv = self.linear(x, w_qkv)
+        self.rope_kv_write(qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache)
+        return qkv
+
     # -- rotation + cache write ----------------------------------------------
     def rope_kv_write(self, qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache):
         N = qkv.shape[0]
