@@ -216,3 +216,32 @@ SIA_EXPORT int sia_cast(const void* in, void* out, long long n, int in_dtype, hi
         return SIA_BAD_ARGUMENT;
     return SIA_LAUNCH_CHECK();
 }
+
+// out[m][k] = scaled[m][k] * rsqrt(sum_p partials[p][m] / width + eps): finishes the norm that a product with a
+// residual epilogue left unfinished, for a consumer that cannot scale its own rows.
+__global__ __launch_bounds__(256) void scale_rows_kernel(const bf16_t* __restrict__ scaled,
+                                                         const float* __restrict__ partials, bf16_t* __restrict__ out,
+                                                         int width, int n_partials, float eps) {
+    __shared__ float sums[256];
+    const int m = blockIdx.x;
+    float ss = 0.f;
+    for (int p = threadIdx.x; p < n_partials; p += 256) ss += partials[p * 16 + m];
+    sums[threadIdx.x] = ss;
+    __syncthreads();
+    for (int half = 128; half > 0; half >>= 1) {
+        if ((int)threadIdx.x < half) sums[threadIdx.x] += sums[threadIdx.x + half];
+        __syncthreads();
+    }
+    const float rs = rsqrtf(sums[0] / (float)width + eps);
+    for (int k = threadIdx.x; k < width; k += 256)
+        out[(size_t)m * width + k] = float_to_bf16(bf16_to_float(scaled[(size_t)m * width + k]) * rs);
+}
+
+SIA_EXPORT int sia_scale_rows(const void* scaled, const float* partials, void* out, int rows, int width,
+                              int n_partials, float eps, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (rows > 16 || width <= 0 || n_partials <= 0) return SIA_BAD_ARGUMENT;
+    hipLaunchKernelGGL(scale_rows_kernel, dim3(rows), dim3(256), 0, stream, (const bf16_t*)scaled, partials,
+                       (bf16_t*)out, width, n_partials, eps);
+    return SIA_LAUNCH_CHECK();
+}

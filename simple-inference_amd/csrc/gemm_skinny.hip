@@ -25,7 +25,7 @@ __device__ __forceinline__ bf16x8 ld8(const bf16_t* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
 
-enum SkinnyEpilogue { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_ROPE = 2 };
+enum SkinnyEpilogue { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_ROPE = 2, EPI_RESIDUAL = 3 };
 
 // What the q/k/v product needs to rotate its result and to put keys and values into the cache pages.
 struct RopeOut {
@@ -39,6 +39,27 @@ struct RopeOut {
     int table_width, n_heads, n_kv, head_dim, page_size;
 };
 
+// The product adds its result into the float residual and leaves what the norm after it needs.
+struct ResidualOut {
+    float* residual;      // [M][N], updated in place
+    const float* gain;    // [N], the norm's weight
+    bf16_t* scaled;       // [M][N] = residual * gain, not yet divided by the row's root mean square
+    float* partials;      // [N / 16][16]: sum over 16 columns of residual^2, by row
+};
+
+// X is such a `scaled` matrix: row m of the result is to be multiplied by rsqrt(sum_p partials[p][m] / K + eps).
+struct RowScale {
+    const float* partials;
+    int n_partials;
+    float eps;
+};
+
+struct Epilogue {
+    RopeOut rope;
+    ResidualOut res;
+    RowScale scale;
+};
+
 // RB: blocks of 16 rows of W per workgroup; WAVES: waves that split K; UNROLL: steps whose loads are in flight
 // together.
 //   EPI_STORE:   row block rb holds rows n0 + 16 rb ..: Y[m][n0 + 16 rb + n]  (TOut)
@@ -48,12 +69,18 @@ struct RopeOut {
 //                the first half of a head and the 16 that the rotation pairs them with (head_dim / 2 further).
 //                q and k are rotated in float on the float sums (one rounding; the rotation kernel rotates the
 //                rounded product, so the two paths differ by a rounding); q goes to Y, k and v into the pages.
-template <typename TOut, int RB, int WAVES, int UNROLL, int EPI>
+//   EPI_RESIDUAL: the result, rounded as EPI_STORE rounds it, is added to the float residual; Y is not written.
+//                RMSNorm(x) W^T = rsqrt(mean x^2 + eps) * ((x * gain) W^T): the kernel leaves x * gain and the sums
+//                of squares of its own 16-column blocks, and the product after it (SCALED) adds those up, in an
+//                order that depends on N only, and scales its rows: no kernel of its own for the norm.
+template <typename TOut, int RB, int WAVES, int UNROLL, int EPI, bool SCALED>
 __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                      const bf16_t* __restrict__ W,
                                                                      TOut* __restrict__ Y, int M, int N, int K,
-                                                                     RopeOut rope) {
+                                                                     const Epilogue ep) {
     __shared__ float part[WAVES][RB][16][17];
+    __shared__ float squares[WAVES][16];
+    const RopeOut& rope = ep.rope;
     constexpr int CHUNK = SK_STEP * UNROLL;  // one wave's share of a round
     constexpr int OUT_BLOCKS = EPI == EPI_SWIGLU ? RB / 2 : RB;  // 16-column blocks of Y per workgroup
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
@@ -71,6 +98,30 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
         const int row = EPI == EPI_ROPE ? n0 + rb * rope_half + r
                                         : n0 + (rb % OUT_BLOCKS) * 16 + (rb / OUT_BLOCKS) * N + r;
         w_row[rb] = W + (size_t)row * K + g * 16;
+    }
+
+    // requested before the weights, used after them
+    constexpr int SQ_LANES = WAVES * 4;  // threads per row that add up the sums of squares
+    const int sq_m = lane & 15, sq_l = wave * 4 + (lane >> 4);
+    float sq[4] = {0.f, 0.f, 0.f, 0.f};
+    if (SCALED) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int p = sq_l + i * SQ_LANES;
+            if (p < ep.scale.n_partials) sq[i] = ep.scale.partials[p * 16 + sq_m];
+        }
+    }
+    constexpr int RES_ITER = (RB * 256 + WAVES * SIA_WAVE - 1) / (WAVES * SIA_WAVE);
+    float res_old[RES_ITER], res_gain[RES_ITER];
+    if (EPI == EPI_RESIDUAL) {
+#pragma unroll
+        for (int it = 0; it < RES_ITER; ++it) {
+            const int idx = threadIdx.x + it * WAVES * SIA_WAVE;
+            const int j = idx / 256, m = (idx / 16) % 16, n = idx % 16;
+            const bool live = idx < RB * 256 && m < M;
+            res_old[it] = live ? ep.res.residual[(size_t)m * N + n0 + j * 16 + n] : 0.f;
+            res_gain[it] = live ? ep.res.gain[n0 + j * 16 + n] : 0.f;
+        }
     }
 
     floatx4 acc[RB];
@@ -103,7 +154,22 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) part[wave][rb][r][g * 4 + i] = acc[rb][i];
+    if (SCALED) {
+        float ss = (sq[0] + sq[1]) + (sq[2] + sq[3]);
+        for (int p = sq_l + 4 * SQ_LANES; p < ep.scale.n_partials; p += SQ_LANES) ss += ep.scale.partials[p * 16 + sq_m];
+        ss += __shfl_xor(ss, 16);
+        ss += __shfl_xor(ss, 32);
+        if (lane < 16) squares[wave][lane] = ss;
+    }
     __syncthreads();
+    // the row's scale: every thread that finishes an element of row m adds the waves' sums in the same order
+    auto row_scale = [&](int m) -> float {
+        if (!SCALED) return 1.f;
+        float ss = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) ss += squares[w][m];
+        return rsqrtf(ss / (float)K + ep.scale.eps);
+    };
     if (EPI == EPI_ROPE) {
         const int m = threadIdx.x / 16, n = threadIdx.x % 16;
         if (threadIdx.x >= 256 || m >= M) return;
@@ -113,6 +179,9 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
             a += part[w][0][m][n];
             b += part[w][1][m][n];
         }
+        const float rs = row_scale(m);
+        a *= rs;
+        b *= rs;
         const int j = rope_j0 + n, pos = rope.positions[m];
         const bool is_v = rope_head >= rope.n_heads + rope.n_kv;
         if (!is_v) {
@@ -143,9 +212,32 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
         }
         return;
     }
+    if (EPI == EPI_RESIDUAL) {
+#pragma unroll
+        for (int it = 0; it < RES_ITER; ++it) {
+            const int idx = threadIdx.x + it * WAVES * SIA_WAVE;
+            const int j = idx / 256, m = (idx / 16) % 16, n = idx % 16;
+            if (idx >= RB * 256 || m >= M) continue;  // a whole 16-lane group leaves or stays
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) s += part[w][j][m][n];
+            const float x = res_old[it] + bf16_to_float(float_to_bf16(s * row_scale(m)));
+            const size_t at = (size_t)m * N + n0 + j * 16 + n;
+            ep.res.residual[at] = x;
+            ep.res.scaled[at] = float_to_bf16(x * res_gain[it]);
+            float xx = x * x;
+            xx += __shfl_xor(xx, 1);
+            xx += __shfl_xor(xx, 2);
+            xx += __shfl_xor(xx, 4);
+            xx += __shfl_xor(xx, 8);
+            if (n == 0) ep.res.partials[(blockIdx.x * RB + j) * 16 + m] = xx;
+        }
+        return;
+    }
     for (int idx = threadIdx.x; idx < OUT_BLOCKS * 256; idx += WAVES * SIA_WAVE) {
         const int j = idx / 256, m = (idx / 16) % 16, n = idx % 16;
         if (m >= M) continue;
+        const float rs = row_scale(m);
         if (EPI == EPI_SWIGLU) {
             float gate = 0.f, up = 0.f;
 #pragma unroll
@@ -153,12 +245,14 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
                 gate += part[w][j][m][n];
                 up += part[w][OUT_BLOCKS + j][m][n];
             }
+            gate *= rs;
+            up *= rs;
             Y[(size_t)m * N + n0 + j * 16 + n] = from_float<TOut>(gate / (1.f + expf(-gate)) * up);
         } else {
             float s = 0.f;
 #pragma unroll
             for (int w = 0; w < WAVES; ++w) s += part[w][j][m][n];
-            Y[(size_t)m * N + n0 + j * 16 + n] = from_float<TOut>(s);
+            Y[(size_t)m * N + n0 + j * 16 + n] = from_float<TOut>(s * rs);
         }
     }
 }
@@ -167,11 +261,12 @@ SIA_EXPORT int sia_gemm_skinny_max_rows() { return 16; }
 
 // Shapes measured on an MI355X at 1 to 16 rows (K 2,048 to 14,336): a workgroup should own as many rows of W as
 // still leave some 160 workgroups (X is fetched once per workgroup); two row blocks go with 16 waves.
-template <typename TOut>
-static void launch_skinny(const bf16_t* X, const bf16_t* W, TOut* Y, int M, int N, int K, hipStream_t stream) {
+template <typename TOut, int EPI>
+static void launch_skinny(const bf16_t* X, const bf16_t* W, TOut* Y, int M, int N, int K, const Epilogue& ep,
+                          hipStream_t stream) {
 #define LAUNCH(RB, WAVES, UNROLL)                                                                                \
-    hipLaunchKernelGGL((gemm_skinny_kernel<TOut, RB, WAVES, UNROLL, EPI_STORE>), dim3(N / (16 * RB)),              \
-                       dim3(WAVES * SIA_WAVE), 0, stream, X, W, Y, M, N, K, RopeOut{})
+    hipLaunchKernelGGL((gemm_skinny_kernel<TOut, RB, WAVES, UNROLL, EPI, false>), dim3(N / (16 * RB)),             \
+                       dim3(WAVES * SIA_WAVE), 0, stream, X, W, Y, M, N, K, ep)
     if (N % 64 == 0 && N / 64 >= 160)
         LAUNCH(4, 8, 2);
     else if (N % 32 == 0 && N / 32 >= 160 && K >= 1024)
@@ -189,48 +284,82 @@ SIA_EXPORT int sia_gemm_skinny(const void* X, const void* W, void* Y, int M, int
     if (M <= 0 || N <= 0) return 0;
     if (M > 16 || N % 16 || K % 64 || K <= 0) return SIA_BAD_ARGUMENT;
     if (out_float)
-        launch_skinny<float>((const bf16_t*)X, (const bf16_t*)W, (float*)Y, M, N, K, stream);
+        launch_skinny<float, EPI_STORE>((const bf16_t*)X, (const bf16_t*)W, (float*)Y, M, N, K, Epilogue{}, stream);
     else
-        launch_skinny<bf16_t>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K, stream);
+        launch_skinny<bf16_t, EPI_STORE>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K, Epilogue{}, stream);
+    return SIA_LAUNCH_CHECK();
+}
+
+// residual[M, N] += round_bf16(X W^T); scaled = residual * gain (bfloat16); partials[N / 16][16] = sums of squares of
+// the residual over blocks of 16 columns, by row (rows >= M are not written).  Needs M <= 16, N % 16 == 0,
+// K % 64 == 0.
+SIA_EXPORT int sia_gemm_skinny_residual(const void* X, const void* W, int M, int N, int K, float* residual,
+                                        const float* gain, void* scaled, float* partials, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || N % 16 || K % 64 || K <= 0 || !residual || !gain || !scaled || !partials) return SIA_BAD_ARGUMENT;
+    Epilogue ep{};
+    ep.res = ResidualOut{residual, gain, (bf16_t*)scaled, partials};
+    launch_skinny<bf16_t, EPI_RESIDUAL>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, ep, stream);
     return SIA_LAUNCH_CHECK();
 }
 
 // Y[M, I] = silu(X Wg^T) * (X Wu^T) for W = [Wg; Wu] of 2 I rows.  Needs M <= 16, I % 16 == 0, K % 64 == 0.
+// With `partials` (else null) X is a `scaled` matrix of sia_gemm_skinny_residual and the rows are divided by their
+// root mean square first.
 SIA_EXPORT int sia_gemm_skinny_swiglu(const void* X, const void* W, void* Y, int M, int inter, int K,
-                                      hipStream_t stream) {
+                                      const float* partials, int n_partials, float eps, hipStream_t stream) {
     if (M <= 0 || inter <= 0) return 0;
-    if (M > 16 || inter % 16 || K % 64 || K <= 0) return SIA_BAD_ARGUMENT;
-    if (inter % 32 == 0 && inter / 32 >= 160 && K >= 1024 && M > 4)
-        hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 4, 16, 2, EPI_SWIGLU>), dim3(inter / 32), dim3(16 * SIA_WAVE), 0,
-                           stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, inter, K, RopeOut{});
+    if (M > 16 || inter % 16 || K % 64 || K <= 0 || (partials && n_partials <= 0)) return SIA_BAD_ARGUMENT;
+    Epilogue ep{};
+    ep.scale = RowScale{partials, n_partials, eps};
+    const bool wide = inter % 32 == 0 && inter / 32 >= 160 && K >= 1024 && M > 4;
+#define LAUNCH(RB, WAVES, SCALED)                                                                                  \
+    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, RB, WAVES, 2, EPI_SWIGLU, SCALED>), dim3(inter / (8 * RB)),      \
+                       dim3(WAVES * SIA_WAVE), 0, stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, inter, \
+                       K, ep)
+    if (wide && partials)
+        LAUNCH(4, 16, true);
+    else if (wide)
+        LAUNCH(4, 16, false);
+    else if (partials)
+        LAUNCH(2, 8, true);
     else
-        hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 2, 8, 2, EPI_SWIGLU>), dim3(inter / 16), dim3(8 * SIA_WAVE), 0,
-                           stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, inter, K, RopeOut{});
+        LAUNCH(2, 8, false);
+#undef LAUNCH
     return SIA_LAUNCH_CHECK();
 }
 
 // The q/k/v product of single-token steps with the rotation and the cache write in its epilogue:
 // W = [q heads | k heads | v heads], head_dim % 32 == 0, every dim of a head rotates (tables of head_dim / 2 floats
 // a position).  Rotated q goes to Y[M][(n_heads + 2 n_kv) head_dim] (its k and v columns are not written); rotated
-// k and v go to the pages at each token's position.  Needs M <= 16, K % 64 == 0.
+// k and v go to the pages at each token's position.  Needs M <= 16, K % 64 == 0.  `partials` as above.
 SIA_EXPORT int sia_gemm_skinny_rope(const void* X, const void* W, void* Y, int M, int K, const float* cos_table,
                                     const float* sin_table, const int* positions, const int* seq_of_token,
                                     const int* block_table, int table_width, void* k_pages, void* v_pages,
-                                    int n_heads, int n_kv, int head_dim, int page_size, hipStream_t stream) {
+                                    int n_heads, int n_kv, int head_dim, int page_size, const float* partials,
+                                    int n_partials, float eps, hipStream_t stream) {
     if (M <= 0) return 0;
     if (M > 16 || K % 64 || K <= 0 || head_dim % 32 || head_dim <= 0 || n_heads <= 0 || n_kv <= 0 || page_size <= 0 ||
         table_width <= 0 || !cos_table || !sin_table || !positions || !seq_of_token || !block_table || !k_pages ||
-        !v_pages)
+        !v_pages || (partials && n_partials <= 0))
         return SIA_BAD_ARGUMENT;
     const int heads = n_heads + 2 * n_kv, N = heads * head_dim;
-    const RopeOut rope{cos_table, sin_table, positions, seq_of_token, block_table, (bf16_t*)k_pages, (bf16_t*)v_pages,
-                       table_width, n_heads, n_kv, head_dim, page_size};
+    Epilogue ep{};
+    ep.rope = RopeOut{cos_table, sin_table, positions, seq_of_token, block_table, (bf16_t*)k_pages, (bf16_t*)v_pages,
+                      table_width, n_heads, n_kv, head_dim, page_size};
+    ep.scale = RowScale{partials, n_partials, eps};
     const dim3 grid(heads * (head_dim / 32));
-    if (K >= 1024)
-        hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 2, 16, 2, EPI_ROPE>), grid, dim3(16 * SIA_WAVE), 0, stream,
-                           (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K, rope);
+#define LAUNCH(WAVES, SCALED)                                                                                      \
+    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 2, WAVES, 2, EPI_ROPE, SCALED>), grid, dim3(WAVES * SIA_WAVE), 0, \
+                       stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K, ep)
+    if (K >= 1024 && partials)
+        LAUNCH(16, true);
+    else if (K >= 1024)
+        LAUNCH(16, false);
+    else if (partials)
+        LAUNCH(8, true);
     else
-        hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 2, 8, 2, EPI_ROPE>), grid, dim3(8 * SIA_WAVE), 0, stream,
-                           (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K, rope);
+        LAUNCH(8, false);
+#undef LAUNCH
     return SIA_LAUNCH_CHECK();
 }

@@ -37,9 +37,11 @@ _SIGNATURES = {
     "sia_sample_workspace_bytes": [_c_int],
     "sia_gemm_skinny": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_gemm_skinny_max_rows": [],
-    "sia_gemm_skinny_swiglu": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_gemm_skinny_swiglu": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_ptr],
     "sia_gemm_skinny_rope": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                             _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                             _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_ptr],
+    "sia_gemm_skinny_residual": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "sia_scale_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr],
 }
 
 
@@ -61,6 +63,34 @@ def attention_library_spec(head_dim: int):
 
 class KernelError(RuntimeError):
     pass
+
+
+class PendingProduct:
+    """A part's output that is still to be computed: ``x @ w^T``.  A residual stream takes it for a delta; the norm
+    that follows may hand it to ``linear_into_residual``, anybody else gets the tensor from ``compute()``."""
+
+    __slots__ = ("x", "w", "kernels")
+
+    def __init__(self, x, w, kernels):
+        self.x, self.w, self.kernels = x, w, kernels
+
+    def compute(self):
+        return self.kernels.linear(self.x, self.w)
+
+
+class ScaledRows:
+    """Rows of an RMS norm that are multiplied by the gain but not yet divided by their root mean square:
+    ``norm(x) = rows * rsqrt(sum_p partials[p, m] / width + eps)``.  ``linear``, ``gated_linear`` and ``qkv_to_cache``
+    take them in place of a tensor and scale the rows of their result instead, which is the same product."""
+
+    __slots__ = ("rows", "partials", "eps")
+
+    def __init__(self, rows, partials, eps):
+        self.rows, self.partials, self.eps = rows, partials, eps
+
+    shape = property(lambda self: self.rows.shape)
+    dtype = property(lambda self: self.rows.dtype)
+    device = property(lambda self: self.rows.device)
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -92,6 +122,7 @@ class HipKernels:
         self._device_index = torch.device(device).index or 0
         self.use_mfma_attention = True   # tests switch it off to reach the plain kernel in bfloat16
         self.use_skinny_gemm = True      # few-row bfloat16 products by this package's kernel, not the library
+        self.fuse_norms = True           # few rows: residual add in the product before a norm, row scale in the one after
         self._skinny_rows = self.core.sia_gemm_skinny_max_rows()
 
     def _attn_lib(self, head_dim: int):
@@ -163,6 +194,7 @@ class HipKernels:
     # -- matrix product --------------------------------------------------------
     def linear(self, x, w, out_float32=False):
         """``x [M, K] @ w [N, K]^T`` with float accumulation."""
+        x = self.finish_rows(x)
         self._want(x, "linear input")
         self._want(w, "linear weight")
         if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
@@ -196,17 +228,67 @@ class HipKernels:
 
     def gated_linear(self, x, w_gate_up):
         """``silu(x Wg^T) * (x Wu^T)`` for ``w_gate_up = [Wg; Wu]``: one kernel for few rows, else product + SwiGLU."""
-        self._want(x, "gated linear input")
         self._want(w_gate_up, "gate/up weight")
         M, K = x.shape
         two_i = w_gate_up.shape[0]
         if (self.use_skinny_gemm and x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
                 and M <= self._skinny_rows and two_i % 32 == 0 and K % 64 == 0 and w_gate_up.shape[1] == K):
-            y = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=x.device)
-            self._check(self.core.sia_gemm_skinny_swiglu(_ptr(x), _ptr(w_gate_up), _ptr(y), M, two_i // 2, K,
-                                                         self._stream()), "gemm_skinny_swiglu")
+            rows, partials, n_partials, eps = self._scaled(x)
+            self._want(rows, "gated linear input")
+            y = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=rows.device)
+            self._check(self.core.sia_gemm_skinny_swiglu(_ptr(rows), _ptr(w_gate_up), _ptr(y), M, two_i // 2, K,
+                                                         _ptr(partials), n_partials, eps, self._stream()),
+                        "gemm_skinny_swiglu")
             return y
         return self.swiglu(self.linear(x, w_gate_up))
+
+    # -- a product whose result goes into the residual, and the norm after it ---------
+    def pending_linear(self, x, w):
+        """``linear(x, w)`` as the last product of a part.  For few rows in bfloat16 it is not computed yet: the norm
+        that follows has it computed by ``linear_into_residual``, which saves the norm's own kernel."""
+        if (self.use_skinny_gemm and self.fuse_norms and isinstance(x, torch.Tensor) and x.dim() == 2 and w.dim() == 2
+                and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] == w.shape[1]
+                and 0 < x.shape[0] <= self._skinny_rows and w.shape[0] % 16 == 0 and w.shape[1] % 64 == 0):
+            return PendingProduct(x, w, self)
+        return self.linear(x, w)
+
+    def linear_into_residual(self, pending, residual, gain, eps):
+        """``residual += x @ w^T`` (the product rounded to bfloat16 first, as ``linear`` rounds it) and the rows of
+        the RMS norm of the sum as ``ScaledRows``."""
+        x, w = pending.x, pending.w
+        self._want(x, "linear input", torch.bfloat16)
+        self._want(w, "linear weight", torch.bfloat16)
+        self._want(residual, "residual", torch.float32)
+        self._want(gain, "norm weight", torch.float32)
+        M, K = x.shape
+        N = w.shape[0]
+        if (w.shape[1] != K or tuple(residual.shape) != (M, N) or tuple(gain.shape) != (N,) or M > self._skinny_rows
+                or N % 16 or K % 64):
+            raise KernelError(f"product into the residual does not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, "
+                              f"residual {tuple(residual.shape)}, gain {tuple(gain.shape)}")
+        rows = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        partials = torch.empty((N // 16, 16), dtype=torch.float32, device=x.device)
+        self._check(self.core.sia_gemm_skinny_residual(_ptr(x), _ptr(w), M, N, K, _ptr(residual), _ptr(gain),
+                                                       _ptr(rows), _ptr(partials), self._stream()),
+                    "gemm_skinny_residual")
+        return ScaledRows(rows, partials, float(eps))
+
+    @staticmethod
+    def _scaled(x):
+        """(rows, partials, n_partials, eps) of an input that may be ``ScaledRows``."""
+        if isinstance(x, ScaledRows):
+            return x.rows, x.partials, x.partials.shape[0], x.eps
+        return x, None, 0, 0.0
+
+    def finish_rows(self, x):
+        """The tensor that ``ScaledRows`` stand for (a tensor is returned as it is)."""
+        if not isinstance(x, ScaledRows):
+            return x
+        out = torch.empty_like(x.rows)
+        self._check(self.core.sia_scale_rows(_ptr(x.rows), _ptr(x.partials), _ptr(out), x.rows.shape[0],
+                                             x.rows.shape[1], x.partials.shape[0], x.eps, self._stream()),
+                    "scale_rows")
+        return out
 
     def gemm_generic(self, x, w, out_float32=False):
         """The plain kernel for either dtype (tests compare it with the library product)."""
@@ -279,6 +361,7 @@ class HipKernels:
         if (self.use_skinny_gemm and n_kv_written and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
                 and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 32 == 0 and K % 64 == 0
                 and not ((n_heads + 2 * n_kv_written) * head_dim < 4096 and K > 4096)):
+            x, partials, n_partials, norm_eps = self._scaled(x)
             self._want(x, "q/k/v input")
             self._want(w_qkv, "q/k/v weight")
             width = (n_heads + 2 * n_kv_written) * head_dim
@@ -297,7 +380,8 @@ class HipKernels:
             self._check(self.core.sia_gemm_skinny_rope(
                 _ptr(x), _ptr(w_qkv), _ptr(qkv), M, K, _ptr(cos), _ptr(sin), _ptr(ctx.positions),
                 _ptr(ctx.seq_of_token), _ptr(cache.block_table), cache.block_table.shape[1], _ptr(cache.k_pages),
-                _ptr(cache.v_pages), n_heads, n_kv_written, head_dim, cache.page_size, self._stream()),
+                _ptr(cache.v_pages), n_heads, n_kv_written, head_dim, cache.page_size, _ptr(partials), n_partials,
+                norm_eps, self._stream()),
                 "gemm_skinny_rope")
             return qkv
         qkv = self.linear(x, w_qkv)

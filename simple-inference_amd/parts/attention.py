@@ -58,6 +58,8 @@ class Attention:
         self.w_qkv = None
         self.w_o = None
 
+    takes_scaled_rows = True   # the input goes to ``qkv_to_cache`` only
+
     @property
     def writes_kv(self) -> bool:
         return self.kv_from_layer is None
@@ -92,4 +94,4 @@ class Attention:
             self.position.rotary_dim, cos, sin, ctx, cache)
         out = k.paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, ctx, cache)
-        return k.linear(out, self.w_o)
+        return k.pending_linear(out, self.w_o)   # the norm after it may have it added into the residual

@@ -20,7 +20,15 @@ class PreNormBlock:
         self.feed_forward_norm = feed_forward_norm
 
     def forward(self, stream, ctx, cache):
-        h = self.mixer_norm.forward(stream)
+        h = _normed(self.mixer_norm, self.mixer, stream)
         stream.delta = self.mixer.forward(h, ctx, cache)
-        h = self.feed_forward_norm.forward(stream)
+        h = _normed(self.feed_forward_norm, self.feed_forward, stream)
         stream.delta = self.feed_forward.forward(h, ctx)
+
+
+def _normed(norm, consumer, stream):
+    """The norm's rows for ``consumer``.  A norm that ``gives_scaled_rows`` may leave the division by the root mean
+    square to a consumer that ``takes_scaled_rows`` (one that hands its input to the kernels' products only)."""
+    if getattr(norm, "gives_scaled_rows", False) and getattr(consumer, "takes_scaled_rows", False):
+        return norm.forward(stream, scaled_ok=True)
+    return norm.forward(stream)

@@ -65,10 +65,24 @@ class ResidualStream:
 
     Parts produce deltas in the compute dtype; the sum over the residual is kept
     in float32 in both modes.  The add is fused into the norm that follows it.
+
+    A part may leave its last product uncomputed (an object with ``compute()``, as the kernels'
+    ``pending_linear`` returns): ``raw_delta`` shows it to a norm that can have it computed
+    straight into the residual; ``delta`` computes it for everybody else.
     """
 
-    __slots__ = ("residual", "delta")
+    __slots__ = ("residual", "raw_delta")
 
     def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None):
         self.residual = residual
-        self.delta = delta
+        self.raw_delta = delta
+
+    @property
+    def delta(self):
+        if hasattr(self.raw_delta, "compute"):
+            self.raw_delta = self.raw_delta.compute()
+        return self.raw_delta
+
+    @delta.setter
+    def delta(self, value):
+        self.raw_delta = value

@@ -25,12 +25,23 @@ class RMSNorm:
     def bind(self, tensors):
         self.weight = tensors["weight"]
 
-    def forward(self, stream, rows=None):
+    gives_scaled_rows = True
+
+    def forward(self, stream, rows=None, scaled_ok=False):
         """Adds ``stream.delta`` into ``stream.residual`` and returns the normed rows.
 
         With ``rows`` (int32 indices) only those rows are computed and the residual
         is left as it was: that form ends a forward pass.
+
+        ``scaled_ok``: the caller also takes the rows undivided by their root mean square (the kernels'
+        ``ScaledRows``).  Then a delta that is a product not yet computed is computed into the residual by the
+        product's own kernel, and the product after the norm divides: the norm has no kernel of its own.
         """
+        k = self.env.kernels
+        if scaled_ok and rows is None and hasattr(stream.raw_delta, "compute") and hasattr(k, "linear_into_residual"):
+            out = k.linear_into_residual(stream.raw_delta, stream.residual, self.weight, self.eps)
+            stream.delta = None
+            return out
         out = self.env.kernels.add_rmsnorm(
             stream.residual, stream.delta, self.weight, self.eps, self.env.dtype, rows)
         if rows is None:

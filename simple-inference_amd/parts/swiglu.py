@@ -18,6 +18,8 @@ from .registry import register_feed_forward
 class SwiGLU:
     """params: hidden_size, intermediate_size."""
 
+    takes_scaled_rows = True   # the input goes to ``gated_linear`` only
+
     def __init__(self, params, env):
         self.hidden = int(params["hidden_size"])
         self.inter = int(params["intermediate_size"])
@@ -39,4 +41,4 @@ class SwiGLU:
     def forward(self, h, ctx):
         k = self.env.kernels
         a = k.gated_linear(h, self.w_gate_up)   # the activation is fused into the product where a kernel has it
-        return k.linear(a, self.w_down)
+        return k.pending_linear(a, self.w_down)   # the norm after it may have it added into the residual

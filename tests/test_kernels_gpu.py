@@ -263,6 +263,79 @@ def test_qkv_product_that_rotates_and_writes_the_pages(hip, geom):
     torch.testing.assert_close(c_hip.v_pages.float(), c_two.v_pages.float(), rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("shape", [
+    # rows, hidden, inner (the K of the product into the residual), intermediate of the gated product after it
+    (8, 3072, 8192, 8192), (1, 3072, 3072, 8192), (16, 192, 64, 96), (5, 5120, 1024, 5120), (13, 1088, 2048, 320),
+])
+def test_norm_shared_out_between_the_products_around_it(hip, shape):
+    """Few rows: the product before a norm adds into the residual and leaves gain * x and sums of squares; the product
+    after it divides its rows by the root mean square.  Compared with product, add + norm and product one by one."""
+    from simple_inference_amd.kernels import PendingProduct, ScaledRows
+    rows, hidden, inner, inter = shape
+    eps = 1e-5
+    x = rnd(rows, inner, dtype=torch.bfloat16, seed=1)
+    w = rnd(hidden, inner, dtype=torch.bfloat16, seed=2, scale=inner ** -0.5)
+    res = rnd(rows, hidden, seed=3, scale=3.0)
+    res[0] *= 40.0   # rows of very different size: each needs its own scale
+    gain = (rnd(hidden, seed=4, scale=0.3) + 1.0).contiguous()
+    w_gu = rnd(2 * inter, hidden, dtype=torch.bfloat16, seed=5, scale=hidden ** -0.5)
+
+    pending = hip.pending_linear(x, w)
+    assert isinstance(pending, PendingProduct)
+    res_fused = res.clone()
+    scaled = hip.linear_into_residual(pending, res_fused, gain, eps)
+    assert isinstance(scaled, ScaledRows)
+
+    res_plain = res.clone()
+    normed = hip.add_rmsnorm(res_plain, hip.linear(x, w), gain, eps, torch.bfloat16, None)
+    # the residual: same sum unless the plain product went to the library, then a rounding of the delta apart
+    torch.testing.assert_close(res_fused, res_plain, rtol=0, atol=2 ** -7)
+    want = res.double() + (x.double() @ w.double().T)
+    torch.testing.assert_close(res_fused.double(), want, rtol=0, atol=2 ** -6)
+    # what it leaves for the product after it: gain * x rounded once, and the sums of squares
+    assert torch.equal(scaled.rows, (res_fused * gain).to(torch.bfloat16))
+    assert tuple(scaled.partials.shape) == (hidden // 16, 16)
+    sums = scaled.partials[:, :rows].double().sum(0)
+    torch.testing.assert_close(sums, res_fused.double().pow(2).sum(-1), rtol=1e-5, atol=0)
+    rs = torch.rsqrt(sums / hidden + eps)[:, None]
+    normed_rows = scaled.rows.double() * rs   # the rows that the fused products multiply, exactly
+    torch.testing.assert_close(hip.finish_rows(scaled).double(), normed_rows, **tol(torch.bfloat16))
+    torch.testing.assert_close(normed.double(), normed_rows, **tol(torch.bfloat16))
+
+    def mean_error(got, ref):
+        return float((got.double() - ref).abs().mean())
+
+    # the gated product: exact given the rows it multiplies, and as near the exact norm as the plain path is
+    gu = normed_rows @ w_gu.double().T
+    fused = hip.gated_linear(scaled, w_gu)
+    torch.testing.assert_close(fused.double(), torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:],
+                               **tol(torch.bfloat16))
+    exact = want * torch.rsqrt(want.pow(2).mean(-1, keepdim=True) + eps) * gain.double()
+    gu = exact @ w_gu.double().T
+    ref = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    assert mean_error(fused, ref) <= 1.25 * mean_error(hip.gated_linear(normed, w_gu), ref) + 1e-5
+    torch.testing.assert_close(hip.linear(scaled, w_gu).double(), normed_rows @ w_gu.double().T, **tol(torch.bfloat16))
+
+    # and into the q/k/v product that rotates and writes the pages
+    D, n_kv, ps = 32, 2, 16
+    n_heads = 4
+    w_qkv = rnd((n_heads + 2 * n_kv) * D, hidden, dtype=torch.bfloat16, seed=6, scale=hidden ** -0.5)
+    kv_lens = [7 + 19 * i for i in range(rows)]
+    ctx = Ctx([1] * rows, kv_lens)
+    pages = sum(-(-kv // ps) for kv in kv_lens) + 2
+    c1 = Cache(pages, n_kv, ps, D, torch.bfloat16, kv_lens, seed=4)
+    c2 = Cache(pages, n_kv, ps, D, torch.float32, kv_lens, seed=4)
+    ang = torch.outer(torch.arange(max(kv_lens) + 1, dtype=torch.float32),
+                      1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)))
+    cos, sin = ang.cos().to(DEV), ang.sin().to(DEV)
+    q1 = hip.qkv_to_cache(scaled, w_qkv, n_heads, n_kv, D, D, cos, sin, ctx, c1)
+    q2 = (normed_rows @ w_qkv.double().T).float()
+    twin.rope_kv_write(q2, n_heads, n_kv, D, D, cos, sin, ctx, c2)
+    torch.testing.assert_close(q1[:, :n_heads * D].float(), q2[:, :n_heads * D], **tol(torch.bfloat16))
+    torch.testing.assert_close(c1.k_pages.float(), c2.k_pages, **tol(torch.bfloat16))
+    torch.testing.assert_close(c1.v_pages.float(), c2.v_pages, **tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("geom", [
     # heads, kv heads, head_dim, page_size, window
     (24, 8, 128, 16, None), (32, 8, 64, 64, None), (16, 1, 32, 8, None), (6, 2, 48, 16, 100), (5, 5, 112, 32, 700),

@@ -40,6 +40,8 @@ class TwinKernels:
         y = x.float() @ w.float().T
         return y if out_float32 else y.to(x.dtype)
 
+    pending_linear = linear   # computed at once: the twin's norm always has a kernel of its own
+
     def gated_linear(self, x, w_gate_up):
         return self.swiglu(self.linear(x, w_gate_up))
 
