@@ -426,11 +426,11 @@ class HipKernels:
     def decode_split(n_seqs: int, n_kv_heads: int, kv_bound: int) -> int:
         """Number of workgroups (four waves each) that share the keys of one (sequence, kv head).  The
         kernel deals a sequence's tiles of 32 keys evenly to the waves.  Enough splits are taken to give
-        each of the 256 compute units a workgroup, but no more than leave every wave about four tiles at
-        the longest length the step can hold: measured at 2,304 keys, more and shorter workgroups cost
-        more in start-up and in combining than they gain."""
+        each of the 256 compute units a workgroup, but no more than leave every wave about two tiles at
+        the longest length the step can hold: measured at 2,048 and 8,192 keys, more and shorter workgroups
+        cost more in start-up and in combining than they gain."""
         want = -(-256 // max(1, n_seqs * n_kv_heads))
-        most = max(1, kv_bound // (4 * 4 * 32))
+        most = max(1, kv_bound // (2 * 4 * 32))
         return max(1, min(want, most))
 
     def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):

@@ -13,7 +13,9 @@ import plain_llama as plain
 # Three tiny configurations that differ in every size and option.  A: 2 layers, 4 query / 2 key-value
 # heads of 16, tied head, no frequency scaling, pages of 4.  B: 3 layers, 3 / 1 heads of 32, untied head,
 # llama3 scaling, pages of 8.  C has sizes that are no power of two, a head size that is not
-# hidden / heads, as many key/value heads as query heads, and another scaling.
+# hidden / heads, as many key/value heads as query heads, and another scaling.  D has widths in multiples of
+# 64 and heads of 64: the sizes at which steps of few tokens take the products that rotate and write the cache,
+# add into the residual and share out the norm between them.
 TINY_A = {
     "architectures": ["LlamaForCausalLM"], "model_type": "llama",
     "hidden_size": 64, "intermediate_size": 128, "num_hidden_layers": 2, "vocab_size": 256,
@@ -42,6 +44,16 @@ TINY_C = {
     "max_position_embeddings": 1024, "bos_token_id": 0, "eos_token_id": 5,
     "tie_word_embeddings": True, "torch_dtype": "bfloat16", "hidden_act": "silu",
 }
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 128, "intermediate_size": 192, "num_hidden_layers": 3, "vocab_size": 320,
+    "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 64,
+    "rms_norm_eps": 2e-6, "rope_theta": 100000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 2.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 3.0, "original_max_position_embeddings": 48},
+    "max_position_embeddings": 2048, "bos_token_id": 3, "eos_token_id": 4,
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "hidden_act": "silu",
+}
 
 
 @dataclass
@@ -57,6 +69,7 @@ TINIES = {
     "a": Tiny("a", TINY_A, 4, 0.02, 0.1),
     "b": Tiny("b", TINY_B, 8, 0.05, 0.0),
     "c": Tiny("c", TINY_C, 16, 0.04, 0.2),
+    "d": Tiny("d", TINY_D, 16, 0.06, 0.15),
 }
 
 

@@ -184,3 +184,44 @@ def test_float32_stored_weights_in_the_bfloat16_engine(tmp_path):
     tokens = random_tokens(mcfg.vocab_size, 40, seed=3)
     got = replay(runner, cache, [([(0, tokens[:33], list(range(33)))], []), ([(0, tokens[33:], list(range(7)))], [0])])
     check_against_plain(got, {0: tokens}, folder, "hip-bf16")
+
+
+@pytest.mark.gpu
+def test_few_token_steps_take_the_products_with_fused_epilogues(folders):
+    """Configuration D has the sizes for them: a step of few tokens in bfloat16 runs one product that rotates and
+    writes the cache and two that add into the residual per layer, and no rotation or norm kernel between layers;
+    a step of many tokens runs none of them.  (That their logits agree with the plain implementation is what the
+    other tests of this file check, for D as for the others.)"""
+    tiny = TINIES["d"]
+    runner, cache, mcfg = make_runner(folders["d"], "hip-bf16", tiny.page_size, num_pages=64)
+    core = runner.kernels.core
+    counted = ("sia_gemm_skinny_rope", "sia_gemm_skinny_residual", "sia_gemm_skinny_swiglu", "sia_rope_kv_write",
+               "sia_add_rmsnorm")
+    calls = {name: 0 for name in counted}
+    real = {name: getattr(core, name) for name in counted}
+
+    def counting(name):
+        def call(*args):
+            calls[name] += 1
+            return real[name](*args)
+        return call
+
+    for name in counted:
+        setattr(core, name, counting(name))
+    try:
+        layers = mcfg.num_hidden_layers
+        tokens = random_tokens(mcfg.vocab_size, 40, seed=5)
+        cache.admit("r")
+        runner.run([StepEntry("r", tokens[:37], [36])])       # many tokens: the library's products, separate kernels
+        assert calls["sia_gemm_skinny_rope"] == calls["sia_gemm_skinny_residual"] == 0
+        assert calls["sia_rope_kv_write"] == layers and calls["sia_add_rmsnorm"] == 2 * layers + 1
+        for name in counted:
+            calls[name] = 0
+        runner.run([StepEntry("r", tokens[37:], [2])])        # three tokens
+        assert calls["sia_gemm_skinny_rope"] == layers and calls["sia_gemm_skinny_swiglu"] == layers
+        assert calls["sia_gemm_skinny_residual"] == 2 * layers - 1   # the last product waits for the rows that are wanted
+        assert calls["sia_rope_kv_write"] == 0 and calls["sia_add_rmsnorm"] == 2   # the first norm and the last
+    finally:
+        for name in counted:
+            setattr(core, name, real[name])
+        cache.release("r")
