@@ -5,8 +5,8 @@ The names and meanings follow the keyword arguments of the reference's
 ``max_running``, ``max_seq_len``, ``block_size``, ``num_kv_blocks``,
 ``token_budget``, ``eos_id``, ``warmup``, ``use_prefix_cache`` and
 ``prefix_cache_blocks`` mean what they mean there; ``use_graphs`` is its
-``use_cuda_graphs`` (hipGraph here).  ``chunk_tokens`` and ``dtype`` have no
-counterpart there: the reference prefills whole prompts (``plan.md:811-868``
+``use_cuda_graphs`` (hipGraph here).  ``chunk_tokens``, ``dtype`` and ``run_ahead``
+have no counterpart there: the reference prefills whole prompts (``plan.md:811-868``
 only sketches portions) and has no 32-bit GPU path.
 """
 
@@ -45,6 +45,7 @@ class EngineConfig:
     dtype: str = "bfloat16"               # "bfloat16" (serving kernels) or "float32" (true 32-bit everywhere)
     eos_id: Optional[int] = None          # None → the model configuration's; -1 → never stop on a token
     use_graphs: Optional[bool] = None     # replay decode-only steps from captured hipGraphs; None → on a GPU, yes
+    run_ahead: bool = True                # with graphs: launch the next decode step before this one's tokens are read
     use_prefix_cache: bool = False        # reuse complete pages of equal prompt prefixes
     prefix_cache_blocks: Optional[int] = None
     warmup: bool = False

@@ -7,6 +7,12 @@ of the step function runs them all as one batch, and the sampler turns the retur
 tokens.  ``run`` steps
 until nothing is left.  The reference's step runs two forwards instead, one for whole prompts
 and one for decoded tokens (``serving/engine.py:330-349``).
+
+Running ahead: a decode step's input tokens are the sampler's output of the step before, which is on the
+device.  When it is certain who takes part in the next step whatever tokens come out (everybody decodes,
+nobody reaches ``max_new_tokens``, nobody can be admitted), that step is launched before the host waits for
+this step's tokens, so the GPU works while the host reads, books and plans.  A request that turns out to have
+ended on an end-of-sequence token has then run one token too far; that token is dropped.
 """
 
 from __future__ import annotations
@@ -57,7 +63,10 @@ class Engine:
         if engine_cfg.graphs_wanted():
             from .graphs import GraphedDecode
             self.graphs = GraphedDecode(self)
-        self.stats = {"steps": 0, "tokens_run": 0, "prefill_tokens": 0, "decode_tokens": 0}
+        self.stats = {"steps": 0, "tokens_run": 0, "prefill_tokens": 0, "decode_tokens": 0, "steps_ahead": 0}
+        self._ahead = None   # (requests, their sampled tokens) of a step launched but not yet read
+        self._token_mirrors = None   # two pinned host buffers that sampled tokens are copied into, in turn
+        self._mirror_turn = 0
         if engine_cfg.warmup:
             self.warmup()
 
@@ -110,6 +119,7 @@ class Engine:
         """Drops every request and gives every page and slot back."""
         self.scheduler.waiting.clear()
         self.scheduler.running.clear()
+        self._ahead = None
         self.cache.reset()
         if self.prefix_cache is not None:
             self.prefix_cache.clear()
@@ -156,6 +166,10 @@ class Engine:
     @torch.no_grad()
     def step(self) -> Dict[int, int]:
         """Runs one iteration; returns {request id: token} for every request that emitted one."""
+        if self._ahead is not None:   # this iteration is already on the GPU
+            emitters, tokens = self._ahead
+            self._ahead = None
+            return self._finish_step(emitters, tokens, chain=True)
         self.scheduler.evict_finished()
         plan = self.scheduler.plan_step(self._try_admit)   # admits, too: into steps with room for prompt tokens
         if not plan:
@@ -176,7 +190,8 @@ class Engine:
         self.stats["steps"] += 1
         self.stats["tokens_run"] += sum(n for _, n in plan)
 
-        if self.graphs is not None and self.graphs.can_run(plan):
+        replayed = self.graphs is not None and self.graphs.can_run(plan)
+        if replayed:
             logits = self.graphs.run(entries)
         else:
             logits = self.runner.run(entries)
@@ -185,13 +200,73 @@ class Engine:
             if self.prefix_cache is not None and req.state is RequestState.PREFILL and req.num_computed < req.prompt_len:
                 # pages a prompt has filled so far can be shared from the next step on
                 self.prefix_cache.insert(req.prompt_tokens[:req.num_computed], self.cache.table(0, req.id))
+        if not emitters:
+            return {}
+        tokens = self._sample(logits, emitters, [r.num_generated for r in emitters])
+        return self._finish_step(emitters, tokens, chain=replayed)
+
+    def _sample(self, logits, emitters: List[Request], draw_indices: List[int]):
+        """Samples on the device and starts the copy of the tokens to the host right behind the sampler, so that
+        work launched later does not stand between the tokens and the host.  Returns (device tokens, read) where
+        ``read()`` waits for the copy and gives the tokens as a list."""
+        tokens = self.sampler.sample_on_device(logits, [r.params for r in emitters], draw_indices)
+        if self.device.type != "cuda":
+            return tokens, tokens.tolist
+        if self._token_mirrors is None:
+            rows = max(self.cfg.max_running, self.cfg.chunk_tokens)
+            self._token_mirrors = [(torch.empty(rows, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+                                   for _ in range(2)]
+        self._mirror_turn ^= 1
+        mirror, copied = self._token_mirrors[self._mirror_turn]
+        n = tokens.numel()
+        mirror[:n].copy_(tokens, non_blocking=True)
+        copied.record()
+
+        def read():
+            copied.synchronize()
+            return mirror[:n].tolist()
+        return tokens, read
+
+    def _finish_step(self, emitters: List[Request], tokens, chain: bool) -> Dict[int, int]:
+        """Reads a step's sampled tokens and books them; before it waits for them, launches the next step if
+        ``chain`` (the step was a replayed decode step) and that step is certain."""
+        on_device, read = tokens
+        if chain and self._next_step_is_certain(emitters):
+            self._ahead = self._launch_ahead(emitters, on_device)
         emitted: Dict[int, int] = {}
-        if emitters:
-            tokens = self.sampler.sample(logits, [r.params for r in emitters], [r.num_generated for r in emitters])
-            for req, token in zip(emitters, tokens):
-                self._emit(req, int(token))
-                emitted[req.id] = int(token)
+        for req, token in zip(emitters, read()):
+            if req.state is RequestState.FINISHED:
+                continue   # ended on an end-of-sequence token a step ago; this step ran ahead of that news
+            self._emit(req, int(token))
+            emitted[req.id] = int(token)
         return emitted
+
+    def _next_step_is_certain(self, emitters: List[Request]) -> bool:
+        """True if the step after the one whose tokens are still on the device runs exactly ``emitters``, one token
+        each, whatever those tokens are: all of them decode on, none reaches its ``max_new_tokens`` with the token
+        it is about to get, and nobody can join (no one waits, or every slot is taken)."""
+        if self.graphs is None or not self.cfg.run_ahead:
+            return False
+        sched = self.scheduler
+        if len(sched.running) != len(emitters) or any(a is not b for a, b in zip(sched.running, emitters)):
+            return False
+        if sched.waiting and len(emitters) < sched.max_running:
+            return False
+        return len(emitters) <= self.graphs.buckets[-1] and all(
+            r.state is RequestState.DECODE and r.num_generated + 1 < r.max_new_tokens for r in emitters)
+
+    def _launch_ahead(self, reqs: List[Request], tokens: torch.Tensor):
+        """Launches the decode step that takes ``tokens`` (on the device, one per request) as its input."""
+        entries = [StepEntry(r.id, [0], [0]) for r in reqs]   # the ids come from the device
+        logits = self.graphs.run(entries, device_tokens=tokens)
+        for r in reqs:
+            r.num_computed += 1
+        self.stats["steps"] += 1
+        self.stats["steps_ahead"] += 1
+        self.stats["tokens_run"] += len(reqs)
+        self.stats["decode_tokens"] += len(reqs)
+        # the draw index counts the token that is not booked yet
+        return reqs, self._sample(logits, reqs, [r.num_generated + 1 for r in reqs])
 
     def _emit(self, req: Request, token: int) -> None:
         """Appends a token and moves the request on (reference: ``serving/engine.py:449-460,499-507``)."""

@@ -113,8 +113,9 @@ class GraphedDecode:
         caches = self.cache.layer_caches(ctx.block_tables)
         return _Bucket(size, kv_bound, meta, host, offsets, ctx, caches, pinned)
 
-    def _fill(self, b: _Bucket, entries: List[StepEntry]) -> None:
-        """Takes this step's pages and writes the step's metadata (padding included) into the buffers."""
+    def _fill(self, b: _Bucket, entries: List[StepEntry], device_tokens=None) -> None:
+        """Takes this step's pages and writes the step's metadata (padding included) into the buffers.
+        ``device_tokens`` (int32, one per entry): the token ids, where they are still on the device."""
         size, off, host = b.size, b.offsets, b.host
         cache = self.cache
         if b.copied is not None:
@@ -150,6 +151,8 @@ class GraphedDecode:
                     host[base:base + self.width] = grp.scratch_page
                     b.rows[(g, s)] = "pad"
         b.meta.copy_(b.pinned, non_blocking=True)
+        if device_tokens is not None:
+            b.ctx.token_ids[:n].copy_(device_tokens)
         if b.copied is None:
             b.copied = torch.cuda.Event()
         b.copied.record()
@@ -189,8 +192,14 @@ class GraphedDecode:
                     self.capture(size, kv_bound)
 
     @torch.no_grad()
-    def run(self, entries: List[StepEntry]) -> torch.Tensor:
+    def run(self, entries: List[StepEntry], device_tokens=None) -> torch.Tensor:
+        """Logits ``[len(entries), vocab]`` of a step of single tokens.  With ``device_tokens`` the entries' own
+        token ids are placeholders and the ids are taken from that int32 device tensor, in the entries' order:
+        the sampler's output of the step before, which the host need not have read yet."""
         self.runner._check(entries)
+        if device_tokens is not None and (device_tokens.dtype != torch.int32 or device_tokens.numel() != len(entries)
+                                          or device_tokens.device != self.device):
+            raise ValueError("device_tokens must be one int32 per entry on the engine's device")
         for e in entries:
             if len(e.tokens) != 1 or list(e.want) != [0]:
                 raise ValueError("a replayed step takes one token per request and returns its logits")
@@ -198,7 +207,7 @@ class GraphedDecode:
         longest = max(self.cache.lengths[e.req] for e in entries) + 1
         kv_bound = self.kv_bucket_of(longest)
         b = self._made.get((size, kv_bound)) or self.capture(size, kv_bound)
-        self._fill(b, entries)
+        self._fill(b, entries, device_tokens)
         b.graph.replay()
         self.replays += 1
         return b.logits[:len(entries)]

@@ -146,3 +146,56 @@ def test_random_request_streams_generate_what_each_request_generates_alone(folde
                dict(max_running=16, num_kv_blocks=400, chunk_tokens=512, use_graphs=False, use_prefix_cache=True)):
         got = run(reqs, True, **kw)
         assert [i for i, (a, b) in enumerate(zip(got, alone)) if a != b] == [], kw
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "d"])
+def test_running_a_step_ahead_changes_no_token(folders, name, dtype):
+    """Decode steps launched before the tokens of the step before are read: requests that end on an
+    end-of-sequence token (found a step late), that end by count, that arrive while others decode and that wait
+    for a slot all get the tokens they get without running ahead, sampled ones included, and every page comes
+    back.  A request that has run past its end-of-sequence token keeps its row for one step, and a request that
+    arrives while a step is running ahead joins one step later, so the rows of a step are then not the same in
+    the two runs; in bfloat16, where the choice of kernel by the number of rows shows in the last bits, no
+    request ends on a token here and all arrive before the first step."""
+    tiny = TINIES[name]
+    vocab = tiny.config["vocab_size"]
+    prompts = [random_tokens(vocab, n, seed=80 + i) for i, n in enumerate((5, 23, 9, 31, 14, 3))]
+    first_params = SamplingParams(max_new_tokens=12, temperature=1.0, seed=7)
+    probe = engine(folders[name], tiny, dtype, run_ahead=False, max_running=1)
+    first = probe.add_request(prompts[0], params=first_params)
+    probe.run()
+    first = first.generated
+    # request 0 ends on this token, in the middle of its allowance
+    stop = next((t for i, t in enumerate(first) if 3 <= i < 10 and t not in first[:i]), None)
+    assert stop is not None, first
+    if dtype == "bfloat16":
+        stop = -1
+
+    def stream(run_ahead):
+        eng = engine(folders[name], tiny, dtype, run_ahead=run_ahead, eos_id=stop, max_running=4)
+        params = [first_params,
+                  SamplingParams(max_new_tokens=20, temperature=0.8, top_k=20, top_p=0.9, seed=3),
+                  SamplingParams(max_new_tokens=7, temperature=0.0, ignore_eos=True),
+                  SamplingParams(max_new_tokens=25, temperature=1.1, seed=9, ignore_eos=True),
+                  SamplingParams(max_new_tokens=9, temperature=0.0),
+                  SamplingParams(max_new_tokens=15, temperature=0.6, top_p=0.8, seed=5)]
+        early = 3 if dtype == "float32" else 6
+        reqs = [eng.add_request(p, params=q) for p, q in zip(prompts[:early], params[:early])]
+        steps = 0
+        while eng.has_work():
+            eng.step()
+            steps += 1
+            if steps == 6:    # arrivals while the first three decode: one finds a slot, two wait for one
+                reqs += [eng.add_request(p, params=q) for p, q in zip(prompts[early:], params[early:])]
+            eng.cache.check()
+        assert all(r.state is RequestState.FINISHED for r in reqs)
+        assert eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks()
+        return [r.generated for r in reqs], eng.stats["steps_ahead"]
+
+    plain_way, none_ahead = stream(False)
+    ahead_way, some_ahead = stream(True)
+    assert none_ahead == 0 and some_ahead > 0
+    assert plain_way == ahead_way
+    if stop >= 0:
+        assert plain_way[0][-1] == stop and 4 <= len(plain_way[0]) <= 10   # the end-of-sequence token ended request 0
