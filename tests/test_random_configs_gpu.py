@@ -1,6 +1,7 @@
 """Seeded random configurations of the architecture through trace replay on the GPU, against the plain
 implementation: head sizes in steps of 16, any number of heads and groups, widths and vocabularies that are
-no multiple of anything convenient, every option on and off."""
+no multiple of anything convenient beside widths in multiples of 64 (which steps of few tokens run through the
+products with fused epilogues), every option on and off."""
 
 import random
 
@@ -27,8 +28,8 @@ def random_config(seed):
                    "original_max_position_embeddings": rng.choice([16, 64, 256])}
     return {
         "architectures": ["LlamaForCausalLM"], "model_type": "llama",
-        "hidden_size": rng.choice([40, 72, 100, 136, 200, 264]),
-        "intermediate_size": rng.choice([56, 96, 150, 224, 328]),
+        "hidden_size": rng.choice([40, 72, 100, 128, 136, 192, 200, 264, 320]),
+        "intermediate_size": rng.choice([56, 96, 150, 192, 224, 256, 328]),
         "num_hidden_layers": rng.choice([1, 2, 3]), "vocab_size": rng.choice([97, 257, 500, 1001]),
         "num_attention_heads": n_kv * group, "num_key_value_heads": n_kv, "head_dim": head_dim,
         "rms_norm_eps": rng.choice([1e-5, 1e-6, 3e-4]), "rope_theta": rng.choice([10000.0, 500000.0]),

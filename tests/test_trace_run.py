@@ -69,7 +69,7 @@ def check(got, prompts, folder, tol):
         assert rel_err(mine, ref) <= tol, r
 
 
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "d"])
 def test_replayer_on_cpu(tmp_path, name):
     from simple_inference_amd.replay import TraceReplayer
     from twins import TwinKernels
