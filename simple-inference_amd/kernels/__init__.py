@@ -123,6 +123,7 @@ class HipKernels:
         self.use_mfma_attention = True   # tests switch it off to reach the plain kernel in bfloat16
         self.use_skinny_gemm = True      # few-row bfloat16 products by this package's kernel, not the library
         self.fuse_norms = True           # few rows: residual add in the product before a norm, row scale in the one after
+        self.fuse_rope = True            # few rows: rotation and cache write in the q/k/v product
         self._skinny_rows = self.core.sia_gemm_skinny_max_rows()
 
     def _attn_lib(self, head_dim: int):
@@ -358,7 +359,7 @@ class HipKernels:
         ``[tokens, (n_heads + 2 n_kv_written) head_dim]`` matrix whose q columns hold the rotated queries; its
         k and v columns are not to be read (for few rows one kernel does all three and never writes them)."""
         M, K = x.shape
-        if (self.use_skinny_gemm and n_kv_written and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
+        if (self.use_skinny_gemm and self.fuse_rope and n_kv_written and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
                 and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 32 == 0 and K % 64 == 0
                 and not ((n_heads + 2 * n_kv_written) * head_dim < 4096 and K > 4096)):
             x, partials, n_partials, norm_eps = self._scaled(x)

@@ -205,3 +205,59 @@ def test_generate_with_stats_has_the_reference_names(folder):
     for key in ("ttft_ms", "tpot_ms", "prefill_ms", "decode_tok_s", "total_wall_ms", "total_tok_s", "peak_vram_gb",
                 "prompt_tokens", "new_tokens"):
         assert key in stats
+
+
+class EagerDecode:
+    """Stands in for the replayed graphs on the CPU: runs single-token steps through the step function, and takes
+    the token ids from a tensor when told to, as a replayed graph takes them from the device."""
+
+    def __init__(self, eng):
+        self.runner = eng.runner
+        self.buckets = [eng.cfg.max_running]
+        self.calls_with_device_tokens = 0
+
+    def can_run(self, plan):
+        return 0 < len(plan) <= self.buckets[-1] and all(n == 1 for _, n in plan)
+
+    def run(self, entries, device_tokens=None):
+        if device_tokens is not None:
+            self.calls_with_device_tokens += 1
+            from simple_inference_amd.engine import StepEntry
+            entries = [StepEntry(e.req, [int(t)], e.want) for e, t in zip(entries, device_tokens.tolist())]
+        return self.runner.run(entries)
+
+
+def test_running_ahead_books_the_same_tokens_and_pages(folder):
+    """The engine's bookkeeping when decode steps are launched before the tokens of the step before are read: a
+    request that ends on an end-of-sequence token (it has then run one token too far), ends by count, arrivals
+    that find a slot or wait for one.  Tokens, states and pages are those of an engine that never runs ahead."""
+    first = plain_greedy(folder, PROMPTS[1], 12)
+    stop = next(t for i, t in enumerate(first) if i >= 3 and t not in first[:i])
+
+    def stream(run_ahead):
+        eng = engine(folder, eos_id=stop, run_ahead=run_ahead, max_running=3)
+        eng.graphs = EagerDecode(eng)
+        params = [SamplingParams(max_new_tokens=12), SamplingParams(max_new_tokens=9, temperature=0.9, seed=4, ignore_eos=True),
+                  SamplingParams(max_new_tokens=20, ignore_eos=True), SamplingParams(max_new_tokens=6, temperature=1.2, top_k=30, seed=8),
+                  SamplingParams(max_new_tokens=15, ignore_eos=True)]
+        prompts = [PROMPTS[1], PROMPTS[0], PROMPTS[2], PROMPTS[1][:9], PROMPTS[3][:30]]
+        reqs = [eng.add_request(p, params=q) for p, q in zip(prompts[:2], params[:2])]
+        emitted_by_step = []
+        while eng.has_work():
+            emitted_by_step.append(eng.step())
+            if len(emitted_by_step) == 5:
+                reqs += [eng.add_request(p, params=q) for p, q in zip(prompts[2:], params[2:])]
+            eng.cache.check()
+        assert all(r.state is RequestState.FINISHED for r in reqs)
+        assert eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks()
+        # every token was reported by exactly one step, in order
+        for r in reqs:
+            assert [e[r.id] for e in emitted_by_step if r.id in e] == r.generated
+        return [r.generated for r in reqs], eng.stats["steps_ahead"], eng.graphs.calls_with_device_tokens
+
+    plain_way, none_ahead, _ = stream(False)
+    ahead_way, some_ahead, from_device = stream(True)
+    assert none_ahead == 0 and some_ahead > 5 and from_device == some_ahead
+    assert ahead_way == plain_way
+    assert plain_way[0] == first[:first.index(stop) + 1]          # ended on the end-of-sequence token
+    assert len(plain_way[2]) == 20 and len(plain_way[4]) == 15     # ended by count
