@@ -67,7 +67,7 @@ def build_engine(args, max_batch, total_len):
     if args.block_size:
         kw["block_size"] = args.block_size
     ecfg = EngineConfig(
-        max_running=max_batch, max_seq_len=4096, dtype=args.dtype, chunk_tokens=max(2048, args.prefill_tokens),
+        max_running=max_batch, max_seq_len=max(4096, -(-total_len // 1024) * 1024), dtype=args.dtype, chunk_tokens=max(2048, args.prefill_tokens),
         eos_id=-1, use_graphs=not args.no_graphs, device="cuda:0", **kw)
     ecfg.num_kv_blocks = max_batch * (-(-total_len // ecfg.block_size)) + 8
     engine = Engine.from_random(cfg, seed=args.seed, engine_cfg=ecfg, std=0.02, generate_on_device=True)
@@ -87,6 +87,12 @@ def random_prompt(vocab, n, seed):
     return torch.randint(0, vocab, (n,), generator=g).tolist()
 
 
+def decode_allowance(engine_or_chunk, batch, context):
+    """Tokens a request may decode while the other prompts of its batch are still being run, and two to spare."""
+    chunk = engine_or_chunk if isinstance(engine_or_chunk, int) else engine_or_chunk.cfg.chunk_tokens
+    return batch * (-(-context // chunk)) + 2
+
+
 def measure_decode(engine, batch, context, steps, warmup, seed=0, sampling=(0.0, 0, 1.0)):
     """(seconds per step, mean context over the timed steps) with ``batch`` requests decoding."""
     from simple_inference_amd import SamplingParams
@@ -95,8 +101,8 @@ def measure_decode(engine, batch, context, steps, warmup, seed=0, sampling=(0.0,
     vocab = engine.model.vocab_size
     temperature, top_k, top_p = sampling
     reqs = [engine.add_request(random_prompt(vocab, context, seed + i), params=SamplingParams(
-        temperature=temperature, top_k=top_k, top_p=top_p, seed=seed + i, max_new_tokens=warmup + steps + batch + 2,
-        ignore_eos=True)) for i in range(batch)]
+        temperature=temperature, top_k=top_k, top_p=top_p, seed=seed + i,
+        max_new_tokens=warmup + steps + decode_allowance(engine, batch, context), ignore_eos=True)) for i in range(batch)]
     while any(r.num_generated == 0 for r in reqs):   # prefill every prompt
         engine.step()
     for _ in range(warmup):
@@ -216,7 +222,9 @@ def main(argv=None):
         return stream_workload(args)
     points = [int(p) for p in args.points.split(",") if p]
     max_batch = max([args.batch] + points)
-    total_len = max(args.context + args.warmup + args.steps + max_batch + 2, args.prefill_tokens + 2)
+    chunk = max(2048, args.prefill_tokens)
+    total_len = max(args.context + args.warmup + args.steps + decode_allowance(chunk, max_batch, args.context),
+                    args.prefill_tokens + 2)
     engine, cfg, layers_full = build_engine(args, max_batch, total_len)
     mc = engine.model_cfg
     dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
@@ -240,7 +248,7 @@ def main(argv=None):
             "model": args.preset + "-shape", "layers": mc.num_hidden_layers, "layers_full": layers_full,
             "hidden": mc.hidden_size, "heads": mc.num_attention_heads, "kv_heads": mc.num_key_value_heads,
             "head_dim": mc.head_dim, "intermediate": mc.intermediate_size, "vocab": mc.vocab_size,
-            "global_batch": args.batch, "seq_len": args.context, "context_limit": 4096,
+            "global_batch": args.batch, "seq_len": args.context, "context_limit": engine.cfg.max_seq_len,
             "page_size": engine.cfg.block_size, "graphs": engine.graphs is not None, "parallelism": "single GPU",
             "sampling": "greedy" if args.temperature == 0 else f"T={args.temperature} k={args.top_k} p={args.top_p}",
         },
