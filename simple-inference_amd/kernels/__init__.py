@@ -125,6 +125,34 @@ class HipKernels:
         self.fuse_norms = True           # few rows: residual add in the product before a norm, row scale in the one after
         self.fuse_rope = True            # few rows: rotation and cache write in the q/k/v product
         self._skinny_rows = self.core.sia_gemm_skinny_max_rows()
+        self.blas = self._load_blas()    # the BLAS library called directly; None: its products go through torch
+
+    def _load_blas(self):
+        """The direct way to the vendor's BLAS library, which spares the host most of what a product through torch
+        costs it.  It is a convenience, not a kernel of this package: if it cannot be built, loaded or initialised
+        the products go through torch, to the same library."""
+        try:
+            lib = build.load_library("blas")
+            lib.sia_blas_init.argtypes, lib.sia_blas_init.restype = [], ctypes.c_int
+            lib.sia_blas_mm.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
+            lib.sia_blas_mm.restype = ctypes.c_int
+            with torch.cuda.device(self.device):
+                if lib.sia_blas_init() != 0:
+                    return None
+            return lib
+        except (build.KernelBuildError, OSError, AttributeError):
+            return None
+
+    def _library_product(self, x, w, out_float32):
+        """``x @ w^T`` for bfloat16 operands by the BLAS library, float accumulation."""
+        if self.blas is not None:
+            M, K = x.shape
+            N = w.shape[0]
+            y = torch.empty((M, N), dtype=torch.float32 if out_float32 else torch.bfloat16, device=x.device)
+            if self.blas.sia_blas_mm(_ptr(x), _ptr(w), _ptr(y), M, N, K, int(out_float32), self._stream()) == 0:
+                return y
+        y = torch.mm(x, w.t())
+        return self.cast(y, torch.float32) if out_float32 else y
 
     def _attn_lib(self, head_dim: int):
         """The matrix-core attention kernels for this head size, compiled at first use."""
@@ -211,8 +239,7 @@ class HipKernels:
                 self._check(self.core.sia_gemm_skinny(_ptr(x), _ptr(w), _ptr(y), M, N, K, int(out_float32),
                                                       self._stream()), "gemm_skinny")
                 return y
-            y = torch.mm(x, w.t())  # BLAS library, float accumulation
-            return self.cast(y, torch.float32) if out_float32 else y
+            return self._library_product(x, w, out_float32)
         # True 32-bit product.  A float32-stored matrix meeting bfloat16 activations widens them.
         back = None
         if x.dtype == torch.bfloat16:

@@ -41,6 +41,14 @@ HIPCC_FLAGS = [
 LIBRARIES: Dict[str, Sequence[str]] = {
     "core": ("elementwise.hip", "rope_cache.hip", "attention_generic.hip", "gemm_generic.hip", "gemm_skinny.hip",
              "sampling.hip"),
+    # the vendor's BLAS library called directly (the products of steps of many tokens); optional: without it those
+    # products go through torch
+    "blas": ("library_product.hip",),
+}
+
+# what a library links beside the HIP runtime
+LINK_FLAGS: Dict[str, Sequence[str]] = {
+    "blas": ("-L/opt/rocm/lib", "-lhipblaslt"),
 }
 
 
@@ -55,12 +63,12 @@ def find_hipcc() -> str:
     raise KernelBuildError("hipcc not found (looked at $HIPCC, /opt/rocm/bin/hipcc and PATH)")
 
 
-def _digest(sources: Iterable[Path], defines: Sequence[str]) -> str:
+def _digest(sources: Iterable[Path], defines: Sequence[str], link: Sequence[str] = ()) -> str:
     h = hashlib.sha256()
     for path in list(sources) + sorted(CSRC.glob("*.h")):
         h.update(path.name.encode())
         h.update(path.read_bytes())
-    h.update(" ".join(list(HIPCC_FLAGS) + list(defines)).encode())
+    h.update(" ".join(list(HIPCC_FLAGS) + list(defines) + list(link)).encode())
     return h.hexdigest()[:12]
 
 
@@ -78,7 +86,7 @@ def _writable_dir() -> Path:
 
 
 def library_path(name: str, sources: Sequence[str], defines: Sequence[str] = ()) -> Path:
-    digest = _digest([CSRC / s for s in sources], defines)
+    digest = _digest([CSRC / s for s in sources], defines, LINK_FLAGS.get(name, ()))
     file = f"libsia_{name}_{digest}.so"
     if (LIB_DIR / file).is_file():
         return LIB_DIR / file
@@ -95,7 +103,7 @@ def compile_library(name: str, sources: Sequence[str], defines: Sequence[str] = 
     out.parent.mkdir(parents=True, exist_ok=True)
     tmp = out.with_suffix(f".tmp{os.getpid()}.so")
     cmd = [hipcc, *HIPCC_FLAGS, *[f"-D{d}" for d in defines], f"-I{CSRC}",
-           *[str(CSRC / s) for s in sources], "-o", str(tmp)]
+           *[str(CSRC / s) for s in sources], "-o", str(tmp), *LINK_FLAGS.get(name, ())]
     if verbose:
         print(f"[simple-inference_amd] compiling {name} ({', '.join(sources)}) for {ARCH} ...",
               file=sys.stderr, flush=True)

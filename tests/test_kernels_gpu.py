@@ -156,6 +156,26 @@ def test_gated_linear(hip, shape):
     torch.testing.assert_close(out.double(), ref, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("shape", [(17, 3072, 3072), (512, 5120, 3072), (2048, 16384, 3072), (130, 3072, 8192),
+                                   (33, 1008, 200), (64, 320, 96)])
+def test_library_product_called_directly(hip, shape):
+    """Products of many rows go to the BLAS library without a tensor library between: same results as through torch
+    (it is the same library), against a float64 product, bfloat16 and float results, again on a second call (the
+    kept algorithm)."""
+    M, N, K = shape
+    assert hip.blas is not None, "the direct way to the BLAS library was not built or did not initialise"
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
+    ref = x.double() @ w.double().T
+    for _ in range(2):
+        out = hip.linear(x, w)
+        assert out.dtype == torch.bfloat16
+        torch.testing.assert_close(out.double(), ref, rtol=1e-2, atol=1e-2 * math.sqrt(K / 64))
+        torch.testing.assert_close(out.float(), torch.mm(x, w.t()).float(), rtol=2e-2, atol=2e-2 * math.sqrt(K / 64))
+        wide = hip.linear(x, w, out_float32=True)
+        assert wide.dtype == torch.float32
+        torch.testing.assert_close(wide.double(), ref, rtol=1e-2, atol=1e-2 * math.sqrt(K / 64))
+
+
 def test_float32_product_has_no_reduced_precision(hip):
     """An operand bit below bfloat16 (8 bits) and tf32 (10 bits) resolution must reach the product."""
     K = 8
