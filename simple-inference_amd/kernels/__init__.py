@@ -5,9 +5,10 @@ torch's current stream, with torch tensors as buffers.  It checks on the host th
 operand shapes, dtypes and devices are what the kernels and their grids assume, and
 raises before a launch that would not fit.  There is no other implementation in this
 package: without a GPU or without ``hipcc`` to build a missing library it raises.
-Matrix products of the bfloat16 path go to the BLAS library through ``torch``, as the
-reference's go to its vendor's (``ops/attention.py:128-130``, ``ops/mlp.py:117,128``);
-the 32-bit path uses this package's own float kernel.
+Matrix products of the bfloat16 path with more than 16 rows go to the vendor's BLAS library
+(called directly, or through ``torch`` where that way is not available), as the reference's
+go to its vendor's (``ops/attention.py:128-130``, ``ops/mlp.py:117,128``); products of fewer
+rows and the whole 32-bit path use this package's own kernels.
 """
 
 from __future__ import annotations
