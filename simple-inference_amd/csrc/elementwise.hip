@@ -245,3 +245,21 @@ SIA_EXPORT int sia_scale_rows(const void* scaled, const float* partials, void* o
                        (bf16_t*)out, width, n_partials, eps);
     return SIA_LAUNCH_CHECK();
 }
+
+// dst[dst_rows[i]] = src[src_rows[i]]: token ids that a sampler has left on the device become the input of the
+// next step without a trip through the host.
+__global__ __launch_bounds__(256) void place_tokens_kernel(int* __restrict__ dst, const int* __restrict__ dst_rows,
+                                                           const int* __restrict__ src,
+                                                           const int* __restrict__ src_rows, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[dst_rows[i]] = src[src_rows[i]];
+}
+
+SIA_EXPORT int sia_place_tokens(int* dst, const int* dst_rows, const int* src, const int* src_rows, int n,
+                                hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (!dst || !dst_rows || !src || !src_rows) return SIA_BAD_ARGUMENT;
+    hipLaunchKernelGGL(place_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, dst, dst_rows, src, src_rows,
+                       n);
+    return SIA_LAUNCH_CHECK();
+}

@@ -8,11 +8,13 @@ tokens.  ``run`` steps
 until nothing is left.  The reference's step runs two forwards instead, one for whole prompts
 and one for decoded tokens (``serving/engine.py:330-349``).
 
-Running ahead: a decode step's input tokens are the sampler's output of the step before, which is on the
-device.  When it is certain who takes part in the next step whatever tokens come out (everybody decodes,
-nobody reaches ``max_new_tokens``, nobody can be admitted), that step is launched before the host waits for
-this step's tokens, so the GPU works while the host reads, books and plans.  A request that turns out to have
-ended on an end-of-sequence token has then run one token too far; that token is dropped.
+Running ahead: a decoding request's next input token is the sampler's output of the step before, which is on
+the device.  Who takes part in the next step, and with how many tokens, depends on the sampled tokens only through
+the ends of requests.  So when no request of the step on the GPU can reach ``max_new_tokens`` with the token it is
+about to get, the next step is planned and launched (admission included) before the host waits for those tokens,
+its token ids copied on the device; the GPU works while the host reads, books and plans.  ``step`` still reports one
+step's tokens per call, in order.  A request that turns out to have ended on an end-of-sequence token has then run
+one token too far; that token is dropped, and its slot goes to the next request a step later.
 """
 
 from __future__ import annotations
@@ -64,7 +66,7 @@ class Engine:
             from .graphs import GraphedDecode
             self.graphs = GraphedDecode(self)
         self.stats = {"steps": 0, "tokens_run": 0, "prefill_tokens": 0, "decode_tokens": 0, "steps_ahead": 0}
-        self._ahead = None   # (requests, their sampled tokens) of a step launched but not yet read
+        self._ahead = None   # a step launched but not yet read: (requests that sampled a token, those tokens)
         self._token_mirrors = None   # two pinned host buffers that sampled tokens are copied into, in turn
         self._mirror_turn = 0
         if engine_cfg.warmup:
@@ -113,7 +115,7 @@ class Engine:
         return req
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._ahead is not None
 
     def reset(self) -> None:
         """Drops every request and gives every page and slot back."""
@@ -166,18 +168,31 @@ class Engine:
     @torch.no_grad()
     def step(self) -> Dict[int, int]:
         """Runs one iteration; returns {request id: token} for every request that emitted one."""
-        if self._ahead is not None:   # this iteration is already on the GPU
-            emitters, tokens = self._ahead
-            self._ahead = None
-            return self._finish_step(emitters, tokens, chain=True)
+        launched = self._ahead
+        self._ahead = None
+        if launched is None:
+            launched = self._launch(None)
+            if launched is None:
+                return {}
+        if self._next_step_is_certain(launched[0]):
+            self._ahead = self._launch(launched)   # before the host waits for this step's tokens
+        return self._collect(*launched)
+
+    def _launch(self, before):
+        """Plans a step and puts it on the GPU.  ``before``: the step launched before it whose tokens the host has
+        not read (its decoding requests take their input from its sampled tokens on the device), or None.
+        Returns (requests that sample a token, their tokens), or None if there is nothing to run."""
         self.scheduler.evict_finished()
         plan = self.scheduler.plan_step(self._try_admit)   # admits, too: into steps with room for prompt tokens
         if not plan:
-            return {}
+            return None
         entries, emitters = [], []
         for req, n in plan:
             if req.state is RequestState.DECODE:
-                entries.append(StepEntry(req.id, [req.last_token], [0]))
+                if req.pending:    # its input is still on the device
+                    entries.append(StepEntry(req.id, [0], [0], token_from=req.pending_row))
+                else:
+                    entries.append(StepEntry(req.id, [req.last_token], [0]))
                 emitters.append(req)
                 self.stats["decode_tokens"] += 1
             else:
@@ -188,22 +203,27 @@ class Engine:
                     emitters.append(req)
                 self.stats["prefill_tokens"] += n
         self.stats["steps"] += 1
+        self.stats["steps_ahead"] += before is not None
         self.stats["tokens_run"] += sum(n for _, n in plan)
 
-        replayed = self.graphs is not None and self.graphs.can_run(plan)
-        if replayed:
-            logits = self.graphs.run(entries)
+        device_tokens = before[1][0] if before is not None and before[1] is not None else None
+        if self.graphs is not None and self.graphs.can_run(plan):
+            logits = self.graphs.run(entries, device_tokens)
         else:
-            logits = self.runner.run(entries)
+            logits = self.runner.run(entries, device_tokens)
         for req, n in plan:
             req.num_computed += n
-            if self.prefix_cache is not None and req.state is RequestState.PREFILL and req.num_computed < req.prompt_len:
+            if self.prefix_cache is not None and req.state is RequestState.PREFILL:
                 # pages a prompt has filled so far can be shared from the next step on
                 self.prefix_cache.insert(req.prompt_tokens[:req.num_computed], self.cache.table(0, req.id))
         if not emitters:
-            return {}
-        tokens = self._sample(logits, emitters, [r.num_generated for r in emitters])
-        return self._finish_step(emitters, tokens, chain=replayed)
+            return [], None
+        tokens = self._sample(logits, emitters, [r.num_generated + r.pending for r in emitters])
+        for row, req in enumerate(emitters):
+            req.state = RequestState.DECODE   # a prompt that has just ended decodes from the next step on
+            req.pending += 1
+            req.pending_row = row
+        return emitters, tokens
 
     def _sample(self, logits, emitters: List[Request], draw_indices: List[int]):
         """Samples on the device and starts the copy of the tokens to the host right behind the sampler, so that
@@ -227,14 +247,13 @@ class Engine:
             return mirror[:n].tolist()
         return tokens, read
 
-    def _finish_step(self, emitters: List[Request], tokens, chain: bool) -> Dict[int, int]:
-        """Reads a step's sampled tokens and books them; before it waits for them, launches the next step if
-        ``chain`` (the step was a replayed decode step) and that step is certain."""
-        on_device, read = tokens
-        if chain and self._next_step_is_certain(emitters):
-            self._ahead = self._launch_ahead(emitters, on_device)
+    def _collect(self, emitters: List[Request], tokens) -> Dict[int, int]:
+        """Reads a launched step's sampled tokens and books them."""
         emitted: Dict[int, int] = {}
-        for req, token in zip(emitters, read()):
+        if not emitters:
+            return emitted
+        for req, token in zip(emitters, tokens[1]()):
+            req.pending -= 1
             if req.state is RequestState.FINISHED:
                 continue   # ended on an end-of-sequence token a step ago; this step ran ahead of that news
             self._emit(req, int(token))
@@ -242,36 +261,14 @@ class Engine:
         return emitted
 
     def _next_step_is_certain(self, emitters: List[Request]) -> bool:
-        """True if the step after the one whose tokens are still on the device runs exactly ``emitters``, one token
-        each, whatever those tokens are: all of them decode on, none reaches its ``max_new_tokens`` with the token
-        it is about to get, and nobody can join (no one waits, or every slot is taken)."""
-        if self.graphs is None or not self.cfg.run_ahead:
-            return False
-        sched = self.scheduler
-        if len(sched.running) != len(emitters) or any(a is not b for a, b in zip(sched.running, emitters)):
-            return False
-        if sched.waiting and len(emitters) < sched.max_running:
-            return False
-        return len(emitters) <= self.graphs.buckets[-1] and all(
-            r.state is RequestState.DECODE and r.num_generated + 1 < r.max_new_tokens for r in emitters)
-
-    def _launch_ahead(self, reqs: List[Request], tokens: torch.Tensor):
-        """Launches the decode step that takes ``tokens`` (on the device, one per request) as its input."""
-        entries = [StepEntry(r.id, [0], [0]) for r in reqs]   # the ids come from the device
-        logits = self.graphs.run(entries, device_tokens=tokens)
-        for r in reqs:
-            r.num_computed += 1
-        self.stats["steps"] += 1
-        self.stats["steps_ahead"] += 1
-        self.stats["tokens_run"] += len(reqs)
-        self.stats["decode_tokens"] += len(reqs)
-        # the draw index counts the token that is not booked yet
-        return reqs, self._sample(logits, reqs, [r.num_generated + 1 for r in reqs])
+        """True if the step after the one whose tokens are still on the device can be planned without them: none
+        of its requests reaches ``max_new_tokens`` with the token it is about to get.  (An end-of-sequence token
+        is found out a step late.)"""
+        return bool(self.cfg.run_ahead and emitters) and all(
+            r.num_generated + r.pending < r.max_new_tokens for r in emitters)
 
     def _emit(self, req: Request, token: int) -> None:
         """Appends a token and moves the request on (reference: ``serving/engine.py:449-460,499-507``)."""
-        if req.state is RequestState.PREFILL and self.prefix_cache is not None:
-            self.prefix_cache.insert(req.prompt_tokens, self.cache.table(0, req.id))
         req.generated.append(token)
         if token in self.eos_ids and not req.params.ignore_eos:
             req.eos_hit = True
@@ -279,8 +276,6 @@ class Engine:
             req.state = RequestState.FINISHED
             self.cache.release(req.id)   # pages and slot go back at once; the next step may hand them out
             req.slot = None
-        else:
-            req.state = RequestState.DECODE
 
     def run(self) -> Dict[int, Request]:
         """Steps until every queued request has finished; returns them by id."""

@@ -95,7 +95,7 @@ class GraphedDecode:
 
     def _make(self, size: int, kv_bound: int) -> _Bucket:
         n_groups = len(self.cache.groups)
-        sizes = [size, size, size, size + 1, size, size, size] + [size * self.width] * n_groups
+        sizes = [size, size, size, size + 1, size, size, size] + [size * self.width] * n_groups + [size, size]
         offsets = [0]
         for s in sizes:
             offsets.append(offsets[-1] + s)
@@ -111,11 +111,13 @@ class GraphedDecode:
             n_decode_seqs=size, q_lens=[1] * size, kv_bound=kv_bound)
         ctx.block_tables = [part(7 + g).view(size, self.width) for g in range(n_groups)]
         caches = self.cache.layer_caches(ctx.block_tables)
-        return _Bucket(size, kv_bound, meta, host, offsets, ctx, caches, pinned)
+        bucket = _Bucket(size, kv_bound, meta, host, offsets, ctx, caches, pinned)
+        bucket.moved = (part(7 + n_groups), part(8 + n_groups))   # rows of this step, rows of the tokens on the device
+        return bucket
 
     def _fill(self, b: _Bucket, entries: List[StepEntry], device_tokens=None) -> None:
-        """Takes this step's pages and writes the step's metadata (padding included) into the buffers.
-        ``device_tokens`` (int32, one per entry): the token ids, where they are still on the device."""
+        """Takes this step's pages and writes the step's metadata (padding included) into the buffers.  Entries
+        with ``token_from`` take their token id from that row of ``device_tokens`` (int32, on the device)."""
         size, off, host = b.size, b.offsets, b.host
         cache = self.cache
         if b.copied is not None:
@@ -150,9 +152,16 @@ class GraphedDecode:
                 elif b.rows.get((g, s)) != "pad":
                     host[base:base + self.width] = grp.scratch_page
                     b.rows[(g, s)] = "pad"
+        moved = [(s, e.token_from) for s, e in enumerate(entries) if e.token_from is not None]
+        if moved:
+            n_groups = len(cache.groups)
+            dst, src = (host[off[7 + n_groups + i]:off[8 + n_groups + i]] for i in range(2))
+            dst[:len(moved)] = [s for s, _ in moved]
+            src[:len(moved)] = [r for _, r in moved]
         b.meta.copy_(b.pinned, non_blocking=True)
-        if device_tokens is not None:
-            b.ctx.token_ids[:n].copy_(device_tokens)
+        if moved:
+            self.runner.kernels.place_tokens(b.ctx.token_ids, b.moved[0][:len(moved)], device_tokens,
+                                             b.moved[1][:len(moved)])
         if b.copied is None:
             b.copied = torch.cuda.Event()
         b.copied.record()
@@ -193,13 +202,14 @@ class GraphedDecode:
 
     @torch.no_grad()
     def run(self, entries: List[StepEntry], device_tokens=None) -> torch.Tensor:
-        """Logits ``[len(entries), vocab]`` of a step of single tokens.  With ``device_tokens`` the entries' own
-        token ids are placeholders and the ids are taken from that int32 device tensor, in the entries' order:
-        the sampler's output of the step before, which the host need not have read yet."""
+        """Logits ``[len(entries), vocab]`` of a step of single tokens.  An entry with ``token_from`` holds a
+        placeholder; its token id is that row of ``device_tokens`` (int32, on the device): the sampler's output of
+        the step before, which the host need not have read yet."""
         self.runner._check(entries)
-        if device_tokens is not None and (device_tokens.dtype != torch.int32 or device_tokens.numel() != len(entries)
-                                          or device_tokens.device != self.device):
-            raise ValueError("device_tokens must be one int32 per entry on the engine's device")
+        for e in entries:
+            if e.token_from is not None and (device_tokens is None or device_tokens.dtype != torch.int32
+                                             or not 0 <= e.token_from < device_tokens.numel()):
+                raise ValueError("an entry takes its token from a row of int32 device_tokens that was not given")
         for e in entries:
             if len(e.tokens) != 1 or list(e.want) != [0]:
                 raise ValueError("a replayed step takes one token per request and returns its logits")

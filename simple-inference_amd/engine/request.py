@@ -29,8 +29,10 @@ class Request:
     slot: Optional[int] = None
     num_computed: int = 0            # tokens whose keys and values are in the cache
     cached_prefix_len: int = 0       # prompt tokens taken from pages of an equal prefix
-    generated: List[int] = field(default_factory=list)
+    generated: List[int] = field(default_factory=list)   # the tokens the host has read
     eos_hit: bool = False
+    pending: int = 0                 # tokens sampled on the device that the host has not read yet
+    pending_row: int = -1            # row of the latest of them among its step's sampled tokens
 
     @property
     def prompt_len(self) -> int:
@@ -46,7 +48,7 @@ class Request:
 
     @property
     def context_len(self) -> int:
-        return self.prompt_len + self.num_generated
+        return self.prompt_len + self.num_generated + self.pending
 
     @property
     def last_token(self) -> int:

@@ -29,6 +29,7 @@ class StepEntry:
     req: int                         # the request's id in the cache manager
     tokens: Sequence[int]            # its next tokens, in order
     want: Sequence[int] = field(default_factory=list)  # places among ``tokens`` whose logits are wanted
+    token_from: Optional[int] = None  # the one token is row ``token_from`` of the step's ``device_tokens``; ``tokens`` holds a placeholder
 
 
 class StepRunner:
@@ -61,9 +62,17 @@ class StepRunner:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"wanted place {w} of request {e.req} is outside its {len(e.tokens)} tokens")
 
-    def build_context(self, entries: List[StepEntry]) -> StepContext:
-        """Takes the pages the step needs and lays its metadata out on the device."""
+    def build_context(self, entries: List[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> StepContext:
+        """Takes the pages the step needs and lays its metadata out on the device.  Entries with ``token_from``
+        get their token id from ``device_tokens`` (int32, on the device), by a copy on the device."""
         self._check(entries)
+        from_device = [e for e in entries if e.token_from is not None]
+        if from_device:
+            if device_tokens is None or device_tokens.dtype != torch.int32:
+                raise ValueError("entries take their tokens from the device, but no int32 device_tokens were given")
+            for e in from_device:
+                if len(e.tokens) != 1 or not 0 <= e.token_from < device_tokens.numel():
+                    raise ValueError(f"request {e.req}: a token from the device is one token, at a row of device_tokens")
         cache = self.cache
         n_seqs = len(entries)
         # Sequences that bring one token go first: the kernels treat them apart from longer runs.
@@ -77,8 +86,9 @@ class StepRunner:
         width = max(1, cache.max_table_len([e.req for e in seqs]))
         n_rows = sum(len(e.want) for e in entries)
 
+        n_moved = len(from_device)
         sizes = [n_tokens, n_tokens, n_tokens, n_seqs + 1, n_seqs, n_seqs, max(n_rows, 1)] + \
-                [n_seqs * width] * n_groups
+                [n_seqs * width] * n_groups + [n_moved, n_moved]
         offsets = np.concatenate([[0], np.cumsum(sizes)])
         host = np.empty(int(offsets[-1]), dtype=np.int32)
         tok, pos, sot, cu, kvl, slots, rows = (host[offsets[i]:offsets[i + 1]] for i in range(7))
@@ -108,8 +118,15 @@ class StepRunner:
                 row = cache.table(g, e.req)
                 tab[s, :len(row)] = row
 
+        if n_moved:
+            dst, src = (host[offsets[7 + n_groups + i]:offsets[8 + n_groups + i]] for i in range(2))
+            dst[:] = [first_token[e.req] for e in from_device]
+            src[:] = [e.token_from for e in from_device]
+
         dev = torch.from_numpy(host).to(self.device)
         part = lambda i: dev[int(offsets[i]):int(offsets[i + 1])]
+        if n_moved:
+            self.kernels.place_tokens(part(0), part(7 + n_groups), device_tokens, part(8 + n_groups))
         ctx = StepContext(
             n_tokens=n_tokens, n_seqs=n_seqs,
             token_ids=part(0), positions=part(1), seq_of_token=part(2), cu_q=part(3), kv_len=part(4),
@@ -121,8 +138,8 @@ class StepRunner:
         return ctx
 
     @torch.no_grad()
-    def run(self, entries: List[StepEntry]) -> Optional[torch.Tensor]:
+    def run(self, entries: List[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Runs one step; returns float32 logits ``[wanted, vocab]`` in the order of entries and wants."""
-        ctx = self.build_context(entries)
+        ctx = self.build_context(entries, device_tokens)
         caches = self.cache.layer_caches(ctx.block_tables)
         return self.model.forward(ctx, caches)

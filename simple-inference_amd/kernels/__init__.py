@@ -42,6 +42,7 @@ _SIGNATURES = {
     "sia_gemm_skinny_rope": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
                              _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_ptr],
     "sia_gemm_skinny_residual": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "sia_place_tokens": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "sia_scale_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr],
 }
 
@@ -191,6 +192,16 @@ class HipKernels:
             raise KernelError(f"{what} must have shape {tuple(shape)}, has {tuple(t.shape)}")
 
     # -- embedding -------------------------------------------------------------
+    def place_tokens(self, token_ids, dst_rows, src_tokens, src_rows):
+        """``token_ids[dst_rows[i]] = src_tokens[src_rows[i]]`` (all int32, on the device)."""
+        for t, what in ((token_ids, "token ids"), (dst_rows, "destination rows"), (src_tokens, "source tokens"),
+                        (src_rows, "source rows")):
+            self._want(t, what, torch.int32)
+        if dst_rows.numel() != src_rows.numel():
+            raise KernelError(f"{dst_rows.numel()} destination rows for {src_rows.numel()} source rows")
+        self._check(self.core.sia_place_tokens(_ptr(token_ids), _ptr(dst_rows), _ptr(src_tokens), _ptr(src_rows),
+                                               dst_rows.numel(), self._stream()), "place_tokens")
+
     def embed(self, token_ids, table):
         self._want(token_ids, "token_ids", torch.int32)
         self._want(table, "embedding table")

@@ -19,6 +19,9 @@ class TwinKernels:
     name = "torch-twins"
 
     # -- embedding ---------------------------------------------------------
+    def place_tokens(self, token_ids, dst_rows, src_tokens, src_rows):
+        token_ids[dst_rows.long()] = src_tokens[src_rows.long()]
+
     def embed(self, token_ids, table):
         return table[token_ids.long()].float()
 
