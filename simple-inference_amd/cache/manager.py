@@ -55,7 +55,10 @@ class PagedGroup:
         self.scratch_page = num_pages
         self.allocator = PageAllocator(num_pages)
         self.tables: Dict[int, List[int]] = {}
-        self.versions: Dict[int, int] = {}   # bumped whenever a request's table changes (graph replay skips rows that did not)
+        # a request's entry changes whenever its table does (graph replay skips rows that did not change); the
+        # numbers come from one counter, so an id that is admitted again never meets a number it had before
+        self.versions: Dict[int, int] = {}
+        self._version = 0
         self.k = self.v = None
         if allocate_storage:
             shape_k = (slabs, num_pages + 1, need.num_kv_heads, page_size, need.head_dim)
@@ -76,7 +79,7 @@ class PagedGroup:
     def begin(self, req: int, reserve: int) -> None:
         self.allocator.reserve(req, reserve)
         self.tables[req] = []
-        self.versions[req] = 0
+        self._touch(req)
 
     def extend(self, req: int, start: int, end: int) -> None:
         """Makes the table ready for a step that writes positions ``start .. end-1``."""
@@ -87,10 +90,14 @@ class PagedGroup:
                 if table[idx] >= 0:
                     self.allocator.free_page(req, table[idx], back_to_reservation=True)
                     table[idx] = -1
-                    self.versions[req] += 1
+                    self._touch(req)
         while len(table) < pages_for(end, self.page_size):
             table.append(self.allocator.allocate(req))
-            self.versions[req] += 1
+            self._touch(req)
+
+    def _touch(self, req: int) -> None:
+        self._version += 1
+        self.versions[req] = self._version
 
     def release(self, req: int) -> None:
         self.allocator.release(req)
@@ -182,7 +189,7 @@ class CacheManager:
             for page in shared:
                 g.allocator.share(req, page)
                 g.tables[req].append(page)
-                g.versions[req] += 1
+                g._touch(req)
         self.lengths[req] = len(shared) * self.page_size
         return slot
 

@@ -74,6 +74,33 @@ def test_graph_replay_equals_eager_on_every_replay(folders, dtype):
     assert graphed.graphs.replays >= 15 and len(graphed.graphs._made) >= 2       # buckets 4, 2, 1 as requests end
 
 
+def test_graph_replay_of_many_rows_equals_eager_on_every_replay(folders):
+    """Twenty and more requests: the products of a replayed step then go to the BLAS library, whose launches are
+    captured with this package's.  Every replay's logits against the same step run eagerly on a twin engine, with
+    eager work and synchronisation between the replays (a captured memset would show from the second replay on)."""
+    tiny = TINIES["d"]
+    vocab = tiny.config["vocab_size"]
+    kw = dict(max_running=24, max_seq_len=128, chunk_tokens=64, run_ahead=False)
+    eager = engine(folders["d"], tiny, "bfloat16", use_graphs=False, **kw)
+    graphed = engine(folders["d"], tiny, "bfloat16", use_graphs=True, **kw)
+    prompts = [random_tokens(vocab, 3 + (7 * i) % 19, seed=120 + i) for i in range(22)]
+    for eng in (eager, graphed):
+        for i, p in enumerate(prompts):
+            eng.cache.admit(i)
+            eng.runner.run([StepEntry(i, p, [])])
+    tokens = [random_tokens(vocab, 12, seed=200 + i) for i in range(22)]
+    worst = 0.0
+    for step in range(12):
+        live = list(range(22 - step // 4))        # 22, 21, 20 rows: one bucket, other paddings
+        entries = [StepEntry(i, [tokens[i][step]], [0]) for i in live]
+        want = eager.runner.run(entries)
+        got = graphed.graphs.run(entries)
+        torch.cuda.synchronize()
+        worst = max(worst, rel_err(got, want))
+    assert graphed.graphs.replays == 12 and len(graphed.graphs._made) == 1
+    assert worst <= 1e-2, worst    # the same kernels and library calls, replayed or not
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replay_logits(folders, dtype):
     tiny = TINIES["c"]
