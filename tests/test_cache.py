@@ -231,16 +231,16 @@ def test_a_table_version_never_comes_back():
     """Graph replay keeps a block-table row while (request, version) is what it wrote.  An id that is admitted
     again after its release, with the same history of growth, must not meet a version it had before: its pages
     may be others now."""
-    m = manager([FULL], num_pages=8)
+    m = manager([FULL], num_pages=16)
     seen = set()
-    for _ in range(3):
+    for turn in range(3):
         m.admit(7)
         for n in (1, 3, 2):
             m.extend(7, n)
             v = (7, m.groups[0].versions[7])
             assert v not in seen
             seen.add(v)
-        m.admit(8)          # takes pages in between, so that request 7 gets others next time
-        m.extend(8, 2)
+        m.admit(100 + turn)          # takes pages in between, so that request 7 gets others next time
+        m.extend(100 + turn, 2)
         m.release(7)
     m.check()
