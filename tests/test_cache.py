@@ -231,7 +231,7 @@ def test_a_table_version_never_comes_back():
     """Graph replay keeps a block-table row while (request, version) is what it wrote.  An id that is admitted
     again after its release, with the same history of growth, must not meet a version it had before: its pages
     may be others now."""
-    m = manager([FULL], num_pages=16)
+    m = manager([FULL], num_pages=16, max_running=5)
     seen = set()
     for turn in range(3):
         m.admit(7)
