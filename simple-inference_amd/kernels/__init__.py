@@ -465,13 +465,16 @@ class HipKernels:
     @staticmethod
     def decode_split(n_seqs: int, n_kv_heads: int, kv_bound: int) -> int:
         """Number of workgroups (four waves each) that share the keys of one (sequence, kv head).  The
-        kernel deals a sequence's tiles of 32 keys evenly to the waves.  Enough splits are taken to give
-        each of the 256 compute units a workgroup, but no more than leave every wave about two tiles at
-        the longest length the step can hold: measured at 2,048 and 8,192 keys, more and shorter workgroups
-        cost more in start-up and in combining than they gain."""
-        want = -(-256 // max(1, n_seqs * n_kv_heads))
+        kernel deals a sequence's tiles of 32 keys evenly to the waves.  Splits are taken while they still give
+        every one of the 256 compute units at most one workgroup, in powers of two (which deal the tiles of the
+        usual lengths evenly), and no more than leave every wave about two tiles at the longest length the step
+        can hold.  Measured at 2,048 and 8,192 keys and 1 to 64 sequences: a split that puts a second workgroup
+        on some compute units, or an odd one, costs more than it gains (12 sequences of 8 kv heads: 2 splits
+        26 us, 3 splits 34 us; 24 sequences: 1 split 40 us, 2 splits 48 us)."""
+        fits = max(1, 256 // max(1, n_seqs * n_kv_heads))
         most = max(1, kv_bound // (2 * 4 * 32))
-        return max(1, min(want, most))
+        want = min(fits, most)
+        return 1 << (want.bit_length() - 1)
 
     def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
         lib = self._attn_lib(head_dim)
