@@ -614,7 +614,7 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     do {                                                                                                        \
         PF_FETCH(FREE, (KB) + 2 * STEP_KEYS);                                                                   \
         _Pragma("unroll") for (int p = 0; p < KTILES; ++p) {                                                    \
-            if (KSPLIT == KTILES && p != part) continue; /* a set of waves per tile, or every wave every tile */ \
+            if (p % KSPLIT != part) continue; /* each set of waves its tiles of the step */                     \
             const int my_kb = (KB) + p * TILE;                                                                  \
             if (wave_live && my_kb <= w_last && my_kb <= wave_hi && my_kb + TILE - 1 >= wave_lo)                \
                 compute_from_lds<PF_NQ>(PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), qf, my_kb, lo, hi, scale, m, l, \
