@@ -38,6 +38,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--num-kv-blocks", type=int, default=None, help="cache pages (default: max_running full contexts)")
     ap.add_argument("--chunk-tokens", type=int, default=512, help="most tokens one step runs")
     ap.add_argument("--no-graphs", action="store_true", help="do not replay decode steps from hipGraphs")
+    ap.add_argument("--no-run-ahead", action="store_true",
+                    help="do not launch a step before the tokens of the step before have been read")
     ap.add_argument("--use-prefix-cache", action="store_true")
     ap.add_argument("--stats-json", metavar="FILE", help="write the run's metrics there")
     ap.add_argument("--device", default="cuda:0")
@@ -69,7 +71,7 @@ def main(argv=None) -> int:
     ecfg = EngineConfig(
         max_running=args.max_running, max_seq_len=args.max_seq_len, block_size=args.block_size,
         num_kv_blocks=args.num_kv_blocks, chunk_tokens=args.chunk_tokens, dtype=args.dtype,
-        use_graphs=not args.no_graphs, use_prefix_cache=args.use_prefix_cache, device=args.device)
+        use_graphs=not args.no_graphs, run_ahead=not args.no_run_ahead, use_prefix_cache=args.use_prefix_cache, device=args.device)
     print("Loading model...", file=sys.stderr, flush=True)
     if args.model:
         engine = Engine.from_folder(args.model, ecfg)
