@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import plain_llama as plain
-from helpers import TINIES, random_tokens, rel_err, write_tiny_model
+from helpers import TINIES, TOLERANCE, random_tokens, rel_err, write_tiny_model
 from simple_inference_amd import Engine, EngineConfig, RequestState, SamplingParams
 from simple_inference_amd.engine import StepEntry
 from simple_inference_amd.sampling import uniform_for
@@ -99,6 +99,37 @@ def test_graph_replay_of_many_rows_equals_eager_on_every_replay(folders):
         worst = max(worst, rel_err(got, want))
     assert graphed.graphs.replays == 12 and len(graphed.graphs._made) == 1
     assert worst <= 1e-2, worst    # the same kernels and library calls, replayed or not
+
+
+def test_long_decoding_crosses_the_length_buckets_of_the_graphs(folders):
+    """Decoding from 500 to 1,040 tokens of context: the replayed graphs change from the 512-token bucket to the
+    1,024-token one and on to the last (other attention grids and key splits), and every token stays the one an
+    eager engine gives (float32: greedy tokens are equal; bfloat16, where the splits show in the last bits and a
+    tiny model's greedy choice hangs on them: the logits of the same given tokens stay within rounding)."""
+    tiny = TINIES["d"]
+    vocab = tiny.config["vocab_size"]
+    prompt = random_tokens(vocab, 500, seed=140)
+    kw = dict(max_seq_len=1100, max_running=2, chunk_tokens=256)
+    graphed = engine(folders["d"], tiny, "float32", use_graphs=True, **kw)
+    eager = engine(folders["d"], tiny, "float32", use_graphs=False, **kw)
+    a = graphed.add_request(prompt, max_new_tokens=540)
+    b = eager.add_request(prompt, max_new_tokens=540)
+    graphed.run()
+    eager.run()
+    assert sorted(kv for _, kv in graphed.graphs._made) == [512, 1024, 1100]
+    assert a.generated == b.generated
+
+    graphed = engine(folders["d"], tiny, "bfloat16", use_graphs=True, **kw)
+    eager = engine(folders["d"], tiny, "bfloat16", use_graphs=False, **kw)
+    for eng in (graphed, eager):
+        eng.cache.admit(1)
+        eng.runner.run([StepEntry(1, prompt, [])])
+    given = random_tokens(vocab, 540, seed=141)
+    worst = 0.0
+    for t in given:
+        worst = max(worst, rel_err(graphed.graphs.run([StepEntry(1, [t], [0])]), eager.runner.run([StepEntry(1, [t], [0])])))
+    assert sorted(kv for _, kv in graphed.graphs._made) == [512, 1024, 1100]
+    assert worst <= TOLERANCE["hip-bf16"], worst   # two bfloat16 paths: no further apart than either may be from the plain one
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
