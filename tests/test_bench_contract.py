@@ -38,3 +38,12 @@ def test_flops_and_bytes_of_the_headline_shape():
     assert layers == 28 * 100_663_296 and head == 128256 * 3072
     assert mc.kv_bytes_per_token(2) == 28 * 8 * 128 * 2 * 2
     json.dumps({"ok": True})
+
+
+def test_decode_allowance_covers_the_steps_that_build_the_contexts():
+    """Requests decode while the other prompts of their batch are still run in portions: they may generate one token
+    for every such step on top of the measured ones, or the first of them would end before the measurement does."""
+    import bench
+    assert bench.decode_allowance(2048, 8, 2048) == 8 + 2
+    assert bench.decode_allowance(2048, 8, 8192) == 8 * 4 + 2
+    assert bench.decode_allowance(2048, 64, 2049) == 64 * 2 + 2
