@@ -51,9 +51,10 @@ _ATTN_SIGNATURES = {
     "sia_attn_decode": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                         _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_attn_prefill": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
-                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "sia_attn_prefill_rows": [],
     "sia_attn_prefill_rows_split": [],
+    "sia_attn_prefill_rows_long": [],
     "sia_attn_mfma_head_dim": [],
 }
 
@@ -496,9 +497,11 @@ class HipKernels:
             rows, rows_split = lib.sia_attn_prefill_rows(), lib.sia_attn_prefill_rows_split()
             n_tiles = sum(-(-q // rows) for q in ctx.q_lens[n_dec:])
             n_tiles_split = sum(-(-q // rows_split) for q in ctx.q_lens[n_dec:]) if rows_split else 0
+            rows_long = lib.sia_attn_prefill_rows_long()
+            n_tiles_long = sum(-(-q // rows_long) for q in ctx.q_lens[n_dec:]) if rows_long else 0
             self._check(lib.sia_attn_prefill(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
-                _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_tiles_split, n_heads,
+                _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_tiles_split, n_tiles_long, n_heads,
                 n_kv_heads, cache.page_size, float(scale), window, self._stream()), "attn_prefill")
 
     # -- sampling ------------------------------------------------------------------

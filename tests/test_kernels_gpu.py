@@ -402,6 +402,26 @@ def test_matrix_core_prefill_in_each_workgroup_shape(hip, q_len, kv_len, window)
     torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
 
 
+def test_matrix_core_prefill_in_workgroups_of_256_tokens(hip):
+    """Very many workgroups (128 heads, 2,500 tokens) take the shape of 8 waves of 32 tokens; a second and a third
+    run in the same launch, shorter than a workgroup and a little longer than one, and a window."""
+    n_heads, n_kv, D, ps = 128, 8, 16, 16
+    dtype = torch.bfloat16
+    q_lens, kv_lens = [2500, 40, 300], [2700, 40, 555]
+    ctx = Ctx(q_lens, kv_lens)
+    cache = Cache(sum(-(-kv // ps) for kv in kv_lens) + 8, n_kv, ps, D, dtype, kv_lens, seed=41)
+    cache.k_pages.copy_(rnd(*cache.k_pages.shape, dtype=dtype, seed=42))
+    cache.v_pages.copy_(rnd(*cache.v_pages.shape, dtype=dtype, seed=43))
+    qkv = rnd(ctx.n_tokens, (n_heads + 2 * n_kv) * D, dtype=dtype, seed=44, scale=2.0)
+    lib = hip._attn_lib(D)
+    assert lib.sia_attn_prefill_rows_long() == 256
+    assert sum(-(-q // lib.sia_attn_prefill_rows()) for q in q_lens) * n_heads >= 2400   # the launch takes that shape
+    for window in (None, 700):
+        out = hip.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache)
+        ref = twin.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache)
+        torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
 def test_matrix_core_attention_runs_longer_than_a_block_table_window(hip, monkeypatch):
     """A wave holds 64 block-table entries at a time.  With pages of 64, runs of more than 4,096 keys that
     start in the middle of a page (tiles are 32 keys) must reload the entries at a page's edge: one decoded
