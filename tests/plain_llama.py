@@ -3,7 +3,7 @@
 Whole sequences, no cache, float32 (or float64), one function for each part.  It
 shares no code with the engine: it reads config.json and the safetensors file
 itself and uses only elementary torch operations.  Every function cites the lines
-of the reference (``/root/reference``) whose formula it writes down.  The reference
+of the reference whose formula it writes down.  The reference
 is read, not run.
 
 Where the reference has two variants of one formula that differ only in where they

@@ -54,14 +54,39 @@ def test_llama3_scaling_branches_and_continuity():
     mid = ~short & ~long_
     assert ((scaled[mid] < base[mid]) & (scaled[mid] > base[mid] / 8.0)).all()
 
-    # continuity at both boundaries: at wavelength 16 the middle rule gives f, at 64 it gives f / factor
-    def at_wavelen(wl):
-        f = 2 * math.pi / wl
-        smooth = (64 / wl - 1.0) / (4.0 - 1.0)
-        return (1 - smooth) * f / 8.0 + smooth * f, f
-    mid16, f16 = at_wavelen(16.0)
-    mid64, f64 = at_wavelen(64.0)
-    assert math.isclose(mid16, f16, rel_tol=1e-12) and math.isclose(mid64, f64 / 8.0, rel_tol=1e-12)
+
+def _second_frequency_at_wavelength(inv_freq_fn, wavelen):
+    """The function's own value, as a multiple of the unscaled frequency, for a frequency of exactly this
+    wavelength: with two frequencies the second is theta^(-1/2), so theta = (wavelen / 2 pi)^2 puts it there."""
+    theta = (wavelen / (2 * math.pi)) ** 2
+    f = float(inv_freq_fn(4, theta)[1])
+    assert math.isclose(2 * math.pi / f, wavelen, rel_tol=1e-6)
+    return float(inv_freq_fn(4, theta, LLAMA3)[1]) / f
+
+
+def _check_the_middle_band(inv_freq_fn):
+    ratio = lambda wl: _second_frequency_at_wavelength(inv_freq_fn, wl)
+    # hand values for factor 8, low 1, high 4, original 64: smooth = (64 / wl - 1) / 3 and the result is
+    # ((1 - smooth) / 8 + smooth) f.  wl = 32: smooth 1/3 -> 5/12;  wl = 24: smooth 5/9 -> 11/18.
+    assert math.isclose(ratio(32.0), 5 / 12, rel_tol=1e-6)      # swapped weights would give 17/24
+    assert math.isclose(ratio(24.0), 11 / 18, rel_tol=1e-6)     # swapped: 37/72
+    # the function is continuous at both ends of the band: just inside it agrees with the rule outside
+    d = 1e-5
+    assert ratio(16.0 * (1 - d)) == 1.0
+    assert math.isclose(ratio(16.0 * (1 + d)), 1.0, rel_tol=2e-5)
+    assert math.isclose(ratio(64.0 * (1 - d)), 1 / 8, rel_tol=1e-4)
+    assert math.isclose(ratio(64.0 * (1 + d)), 1 / 8, rel_tol=1e-6)
+
+
+def test_llama3_middle_band_by_hand_values_and_continuity_of_the_function():
+    _check_the_middle_band(plain.rope_inv_freq)
+
+
+def test_the_package_frequencies_obey_the_same_hand_values():
+    from simple_inference_amd.parts.rope import rotary_inv_freq
+    _check_the_middle_band(rotary_inv_freq)
+    for dim, theta in ((32, 500000.0), (48, 25000.0)):
+        assert torch.allclose(rotary_inv_freq(dim, theta, LLAMA3), plain.rope_inv_freq(dim, theta, LLAMA3), rtol=1e-6)
 
 
 def test_rotation_pairs_i_with_i_plus_half():
