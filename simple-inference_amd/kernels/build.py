@@ -2,7 +2,7 @@
 
 Each library is built from one or more ``.hip`` files with ``hipcc`` (no torch headers, so a
 build takes seconds) and loaded with ``ctypes``.  A library's file name carries a hash of
-its sources, of ``common.h`` and of the flags, so a changed source is never served by a
+its sources, of the headers they include and of the flags, so a changed source is never served by a
 stale build.  Libraries are kept beside this file (``_lib/``); if that folder cannot be
 written they go to a per-user folder under the temporary directory.  What is missing is
 compiled at first use, with a progress line per file.
@@ -63,9 +63,24 @@ def find_hipcc() -> str:
     raise KernelBuildError("hipcc not found (looked at $HIPCC, /opt/rocm/bin/hipcc and PATH)")
 
 
+_INCLUDE = re.compile(r'^\s*#\s*include\s+"([^"]+)"', re.M)
+
+
+def _headers_of(sources: Iterable[Path]) -> list:
+    """The headers under ``csrc/`` that the sources include, directly or through one another, sorted by name."""
+    found, todo = {}, list(sources)
+    while todo:
+        for name in _INCLUDE.findall(todo.pop().read_text()):
+            path = CSRC / name
+            if name not in found and path.is_file():
+                found[name] = path
+                todo.append(path)
+    return [found[name] for name in sorted(found)]
+
+
 def _digest(sources: Iterable[Path], defines: Sequence[str], link: Sequence[str] = ()) -> str:
     h = hashlib.sha256()
-    for path in list(sources) + sorted(CSRC.glob("*.h")):
+    for path in list(sources) + _headers_of(sources):
         h.update(path.name.encode())
         h.update(path.read_bytes())
     h.update(" ".join(list(HIPCC_FLAGS) + list(defines) + list(link)).encode())
