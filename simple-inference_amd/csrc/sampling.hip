@@ -25,6 +25,10 @@
 // recomputing, from the histograms of the passes before it, what those passes decided; nothing but the
 // histograms travels between launches.  Launches whose filter no row asks for are skipped by the caller's hint.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <cstddef>
+#include <mutex>
 
 #define SP_CHUNKS 16
 #define SP_THREADS 1024
@@ -374,18 +378,10 @@ __global__ __launch_bounds__(SP_THREADS) void sample_pick_kernel(const float* __
 
 SIA_EXPORT long long sia_sample_workspace_bytes(int rows) { return (long long)rows * (long long)sizeof(SampleRow); }
 
-// One token per row.  workspace: sia_sample_workspace_bytes(rows) bytes, all zero (with filters == 0 they may
-// hold anything).  filters: bit 0 set if
-// some row may have a top-k filter, bit 1 if some row may have a top-p filter in (0, 1), bit 2 if some row has
-// a temperature above 0; launches for filters that no row has are skipped (rows decide for themselves inside
-// the launches that run).  With filters == 0 the parameter pointers may be null: every row takes its argmax.
-SIA_EXPORT int sia_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
-                          const float* uniform, int* out, void* workspace, int rows, int vocab, int filters,
-                          hipStream_t stream) {
-    if (rows <= 0) return 0;
-    if (vocab <= 0 || rows > 65535 || !workspace) return SIA_BAD_ARGUMENT;
-    if (filters && (!temperature || !top_k || !top_p || !uniform)) return SIA_BAD_ARGUMENT;
-    SampleRow* ws = (SampleRow*)workspace;
+// The launches of one call, on a workspace whose histograms are zero.
+static int launch_sampling(const float* logits, const float* temperature, const int* top_k, const float* top_p,
+                           const float* uniform, int* out, SampleRow* ws, int rows, int vocab, int filters,
+                           hipStream_t stream) {
     const dim3 grid(SP_CHUNKS, rows), block(SP_THREADS);
     int bits = 62;  // fixed point: vocab * 2^bits < 2^63
     while (bits > 0 && ((long long)vocab << bits) >> bits != (long long)vocab) --bits;
@@ -405,4 +401,77 @@ SIA_EXPORT int sia_sample(const float* logits, const float* temperature, const i
     hipLaunchKernelGGL(sample_pick_kernel, dim3(rows), block, 0, stream, logits, filters ? temperature : nullptr, top_k,
                        top_p, uniform, out, vocab, ws, one);
     return SIA_LAUNCH_CHECK();
+}
+
+// One token per row.  workspace: sia_sample_workspace_bytes(rows) bytes, all zero (with filters == 0 they may
+// hold anything).  filters: bit 0 set if
+// some row may have a top-k filter, bit 1 if some row may have a top-p filter in (0, 1), bit 2 if some row has
+// a temperature above 0; launches for filters that no row has are skipped (rows decide for themselves inside
+// the launches that run).  With filters == 0 the parameter pointers may be null: every row takes its argmax.
+SIA_EXPORT int sia_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
+                          const float* uniform, int* out, void* workspace, int rows, int vocab, int filters,
+                          hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0 || rows > 65535 || !workspace) return SIA_BAD_ARGUMENT;
+    if (filters && (!temperature || !top_k || !top_p || !uniform)) return SIA_BAD_ARGUMENT;
+    return launch_sampling(logits, temperature, top_k, top_p, uniform, out, (SampleRow*)workspace, rows, vocab, filters,
+                           stream);
+}
+
+// ---- the same, for callers that cannot allocate -------------------------------------------------------------
+// The workspace is a fixed array in device memory that belongs to this library: SIA_SAMPLE_STATIC_MAX_ROWS rows
+// (about 4.5 MiB on every GPU the library is used on, until the process ends).  Host code never passes the
+// array's name to a kernel: the name is a host-side stand-in, and each GPU holds a copy of its own, so the device
+// address is asked for once per device, with that device current, and kept.
+static __device__ __align__(256) unsigned char scratch[SIA_SAMPLE_STATIC_MAX_ROWS * sizeof(SampleRow)];
+
+#define SIA_MAX_DEVICES 64
+static void* scratch_on_device[SIA_MAX_DEVICES];
+static std::mutex scratch_guard;
+
+// Device address of `scratch` on the current device.
+static int scratch_address(SampleRow** out) {
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return (int)err;
+    if (device < 0 || device >= SIA_MAX_DEVICES) return SIA_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> hold(scratch_guard);
+    if (!scratch_on_device[device]) {
+        void* ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return (int)err;
+        if (!ptr) return SIA_BAD_ARGUMENT;
+        scratch_on_device[device] = ptr;
+    }
+    *out = (SampleRow*)scratch_on_device[device];
+    return 0;
+}
+
+// Zeroes the histograms (the leading members of SampleRow) of the first rows of a workspace.  A kernel, not a
+// memset: a caller may be recording a graph, and fill nodes are not reliable in replayed graphs.
+#define SP_CLEAR_BYTES (sizeof(u64) * SP_PASSES * SP_MAX_BINS + sizeof(int) * SP_PASSES * SP_MAX_BINS)
+static_assert(offsetof(SampleRow, kept) == SP_CLEAR_BYTES, "the histograms lead the row and are contiguous");
+static_assert(SP_CLEAR_BYTES % sizeof(uint4) == 0 && sizeof(SampleRow) % sizeof(uint4) == 0, "cleared in 16-byte pieces");
+__global__ __launch_bounds__(SP_THREADS) void sample_clear_kernel(SampleRow* __restrict__ ws) {
+    const int piece = blockIdx.x * SP_THREADS + threadIdx.x;
+    if (piece < (int)(SP_CLEAR_BYTES / sizeof(uint4))) ((uint4*)(ws + blockIdx.y))[piece] = make_uint4(0, 0, 0, 0);
+}
+
+SIA_EXPORT int sia_sample_static_max_rows(void) { return SIA_SAMPLE_STATIC_MAX_ROWS; }
+
+SIA_EXPORT int sia_sample_static(const float* logits, const float* temperature, const int* top_k, const float* top_p,
+                                 const float* uniform, int* out, int rows, int vocab, int filters,
+                                 hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0 || rows > SIA_SAMPLE_STATIC_MAX_ROWS) return SIA_BAD_ARGUMENT;
+    if (filters && (!temperature || !top_k || !top_p || !uniform)) return SIA_BAD_ARGUMENT;
+    SampleRow* ws = nullptr;
+    const int err = scratch_address(&ws);
+    if (err) return err;
+    if (filters) {  // the last call's histograms are still there
+        const int pieces = (int)(SP_CLEAR_BYTES / sizeof(uint4));
+        hipLaunchKernelGGL(sample_clear_kernel, dim3((pieces + SP_THREADS - 1) / SP_THREADS, rows), dim3(SP_THREADS), 0,
+                           stream, ws);
+    }
+    return launch_sampling(logits, temperature, top_k, top_p, uniform, out, ws, rows, vocab, filters, stream);
 }
