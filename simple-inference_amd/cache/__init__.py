@@ -1,5 +1,5 @@
-from .allocator import PageAllocator
+from .allocator import OutOfPages, PagePool
 from .manager import CacheManager, PagedGroup, StateSlots, pages_for
 from .prefix import PrefixCache
 
-__all__ = ["PageAllocator", "CacheManager", "PagedGroup", "StateSlots", "pages_for", "PrefixCache"]
+__all__ = ["OutOfPages", "PagePool", "CacheManager", "PagedGroup", "StateSlots", "pages_for", "PrefixCache"]

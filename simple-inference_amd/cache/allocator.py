@@ -1,143 +1,196 @@
-"""Page ids: who holds them, how many are promised, which are free.
+"""The pool of page ids of one cache group: who holds which page, and what is promised to whom.
 
-Same contract as the reference's ``BlockAllocator`` (``serving/block_allocator.py:22-140``):
-a min-heap of free ids (lowest id first), a reference count per page, and a
-per-owner *reservation* (pages promised but not yet handed out) with the
-invariant ``free - reserved >= 0``.  Beyond the reference:
+The contract is that of the reference's block allocator (``serving/block_allocator.py:22-140``):
+pages are handed out lowest id first, a page may have several holders and is free again when the
+last one lets go, and an owner can be *promised* pages in advance, which nobody else can then take
+(the pool never promises more than it has free).  The bookkeeping is this package's own:
 
-* ``allocate`` also serves an owner whose reservation is used up (or was zero),
-  from pages that nobody has been promised; trace replay allocates that way,
-  because it does not know a request's length in advance.
-* ``free_page`` gives one page back early (a window has passed it) and can put
-  it back into the owner's reservation.
+* Ids that were never handed out lie above a watermark; only ids that came back are kept in a
+  heap.  A pool of hundreds of thousands of pages costs nothing to set up, and "lowest first"
+  holds because every id below the watermark that is free is in the heap.
+* Owners have *accounts* (``open`` .. ``close``).  An account whose promise is used up, or that
+  was opened without one, may still ``take`` pages that are promised to nobody: trace replay
+  works that way, because it does not know a request's length in advance.
+* A page can also be held without an account (``pin`` / ``unpin``): the prefix cache keeps
+  pages alive that way after the request that wrote them has gone.
+* ``drop`` gives one page back early (a window has passed it) and can turn it back into a
+  promise, so that a windowed request can never run dry.
 """
 
 from __future__ import annotations
 
 import heapq
-from typing import Dict, List, Set
+from typing import Dict, FrozenSet, List, Set
 
 
-class PageAllocator:
+class OutOfPages(MemoryError):
+    """The pool cannot promise or hand out what was asked."""
+
+
+class _Account:
+    __slots__ = ("promised", "pages")
+
+    def __init__(self, promised: int):
+        self.promised = promised      # pages this owner may still take for certain
+        self.pages: Set[int] = set()
+
+
+class PagePool:
     def __init__(self, num_pages: int):
         if num_pages <= 0:
-            raise ValueError(f"num_pages must be positive, got {num_pages}")
+            raise ValueError(f"a pool needs at least one page, got {num_pages}")
         self.num_pages = num_pages
-        self._free: List[int] = list(range(num_pages))
-        heapq.heapify(self._free)
-        self._refs = [0] * num_pages
-        self._reserved: Dict[int, int] = {}
-        self._owned: Dict[int, Set[int]] = {}
+        self._fresh = 0                      # ids at or above it were never handed out
+        self._returned: List[int] = []       # heap of free ids below the watermark
+        self._holders = [0] * num_pages      # accounts plus pins holding each page
+        self._pins: Dict[int, int] = {}
+        self._accounts: Dict[int, _Account] = {}
+        self._promised = 0                   # sum of the accounts' open promises
 
-    # -- counts ------------------------------------------------------------
+    # -- counts --------------------------------------------------------------------------
     @property
-    def free_pages(self) -> int:
-        return len(self._free)
-
-    @property
-    def reserved_pages(self) -> int:
-        return sum(self._reserved.values())
+    def n_free(self) -> int:
+        return self.num_pages - self._fresh + len(self._returned)
 
     @property
-    def available_pages(self) -> int:
-        """Free pages that are promised to nobody."""
-        return self.free_pages - self.reserved_pages
+    def n_promised(self) -> int:
+        return self._promised
 
-    def ref_count(self, page: int) -> int:
-        self._check_id(page)
-        return self._refs[page]
+    @property
+    def n_unpromised(self) -> int:
+        """Free pages that nobody has been promised."""
+        return self.n_free - self._promised
 
-    def owners(self):
-        return list(self._owned)
+    def holders(self, page: int) -> int:
+        return self._holders[self._valid(page)]
 
-    def pages_of(self, owner: int) -> Set[int]:
-        return set(self._owned.get(owner, ()))
+    def fits(self, promise: int) -> bool:
+        return 0 <= promise <= self.n_unpromised
 
-    # -- reservations ------------------------------------------------------
-    def can_reserve(self, owner: int, count: int) -> bool:
-        if owner in self._reserved:
-            raise ValueError(f"owner {owner} already has a reservation")
-        return 0 <= count <= self.available_pages
+    # -- accounts ------------------------------------------------------------------------
+    def has(self, owner: int) -> bool:
+        return owner in self._accounts
 
-    def reserve(self, owner: int, count: int) -> None:
-        if count < 0:
-            raise ValueError(f"count must be non-negative, got {count}")
-        if not self.can_reserve(owner, count):
-            raise MemoryError(f"cannot reserve {count} pages for owner {owner}: {self.available_pages} remain")
-        self._reserved[owner] = count
-        self._owned[owner] = set()
+    def owners(self) -> List[int]:
+        return list(self._accounts)
 
-    # -- pages -------------------------------------------------------------
-    def allocate(self, owner: int) -> int:
-        if owner not in self._reserved:
-            raise KeyError(f"owner {owner} has no reservation")
-        if self._reserved[owner] > 0:
-            if not self._free:
-                raise RuntimeError("reservation invariant violated: no free page for a reserved owner")
-            self._reserved[owner] -= 1
-        elif self.available_pages <= 0:
-            raise MemoryError(f"owner {owner} has used its reservation and no unpromised page is free")
-        page = heapq.heappop(self._free)
-        self._refs[page] = 1
-        self._owned[owner].add(page)
+    def pages(self, owner: int) -> FrozenSet[int]:
+        acct = self._accounts.get(owner)
+        return frozenset(acct.pages) if acct else frozenset()
+
+    def open(self, owner: int, promise: int = 0) -> None:
+        if owner in self._accounts:
+            raise ValueError(f"owner {owner} has an account already")
+        if promise < 0:
+            raise ValueError(f"a promise cannot be negative ({promise})")
+        if promise > self.n_unpromised:
+            raise OutOfPages(f"{promise} pages cannot be promised to owner {owner}: {self.n_unpromised} are unpromised")
+        self._accounts[owner] = _Account(promise)
+        self._promised += promise
+
+    def close(self, owner: int) -> None:
+        """Lets go of every page of the owner and of what is left of its promise; an unknown owner is ignored."""
+        acct = self._accounts.pop(owner, None)
+        if acct is None:
+            return
+        self._promised -= acct.promised
+        for page in acct.pages:
+            self._let_go(page)
+
+    # -- pages ---------------------------------------------------------------------------
+    def take(self, owner: int) -> int:
+        """The lowest free page, against the owner's promise while it lasts, else from the unpromised ones."""
+        acct = self._account(owner)
+        if acct.promised:
+            if not self.n_free:
+                raise RuntimeError("a promised page is missing: more was promised than is free")
+            acct.promised -= 1
+            self._promised -= 1
+        elif self.n_unpromised <= 0:
+            raise OutOfPages(f"owner {owner} holds no promise and every free page is promised to someone")
+        if self._returned:
+            page = heapq.heappop(self._returned)
+        else:
+            page = self._fresh
+            self._fresh += 1
+        self._holders[page] = 1
+        acct.pages.add(page)
         return page
 
-    def share(self, owner: int, page: int) -> None:
-        """Adds an existing page to another owner (reference: ``incref``)."""
-        self._check_id(page)
-        if owner not in self._reserved:
-            raise KeyError(f"owner {owner} has no reservation")
-        if page in self._owned[owner]:
-            raise ValueError(f"owner {owner} already holds page {page}")
-        if self._refs[page] == 0:
-            raise ValueError(f"cannot share free page {page}")
-        self._refs[page] += 1
-        self._owned[owner].add(page)
+    def adopt(self, owner: int, page: int) -> None:
+        """Makes the owner one more holder of a page that is in use (the reference's ``incref``)."""
+        acct = self._account(owner)
+        if page in acct.pages:
+            raise ValueError(f"owner {owner} holds page {page} already")
+        if not self._holders[self._valid(page)]:
+            raise ValueError(f"page {page} is free and cannot be adopted")
+        self._holders[page] += 1
+        acct.pages.add(page)
 
-    def free_page(self, owner: int, page: int, back_to_reservation: bool = False) -> None:
-        if owner not in self._owned or page not in self._owned[owner]:
+    def drop(self, owner: int, page: int, restore_promise: bool = False) -> None:
+        """The owner lets go of one page; with ``restore_promise`` it may take one page more for certain later."""
+        acct = self._accounts.get(owner)
+        if acct is None or page not in acct.pages:
             raise KeyError(f"owner {owner} does not hold page {page}")
-        self._owned[owner].remove(page)
-        self._decref(page)
-        if back_to_reservation:
-            if self.available_pages <= 0:
-                raise RuntimeError("reservation invariant violated while returning a page to a reservation")
-            self._reserved[owner] += 1
+        acct.pages.discard(page)
+        self._let_go(page)
+        if restore_promise:
+            if self.n_unpromised <= 0:
+                raise RuntimeError("no unpromised page is left to turn back into a promise")
+            acct.promised += 1
+            self._promised += 1
 
-    def release(self, owner: int) -> None:
-        """Drops every page and the reservation of an owner; unknown owners are ignored."""
-        owned = self._owned.pop(owner, None)
-        if owned is None:
-            return
-        for page in owned:
-            self._decref(page)
-        self._reserved.pop(owner)
+    def pin(self, page: int) -> None:
+        """One more holder of a page in use, outside every account."""
+        if not self._holders[self._valid(page)]:
+            raise ValueError(f"page {page} is free and cannot be pinned")
+        self._holders[page] += 1
+        self._pins[page] = self._pins.get(page, 0) + 1
 
-    # -- checks ------------------------------------------------------------
-    def check(self) -> None:
-        """No page lost, none held twice by one owner, none free while held."""
-        free = set(self._free)
-        if len(free) != len(self._free):
-            raise AssertionError("a page is in the free list twice")
-        counts = [0] * self.num_pages
-        for pages in self._owned.values():
-            for p in pages:
-                counts[p] += 1
+    def unpin(self, page: int) -> None:
+        left = self._pins.get(self._valid(page), 0) - 1
+        if left < 0:
+            raise KeyError(f"page {page} is not pinned")
+        if left:
+            self._pins[page] = left
+        else:
+            del self._pins[page]
+        self._let_go(page)
+
+    # -- checks --------------------------------------------------------------------------
+    def audit(self) -> None:
+        """Every page is free or held, exactly as often as its count says; nothing is promised that is not there."""
+        free = set(self._returned) | set(range(self._fresh, self.num_pages))
+        if len(free) != self.n_free or any(p >= self._fresh for p in self._returned):
+            raise AssertionError("a page is in the free set twice")
+        seen = [self._pins.get(p, 0) for p in range(self.num_pages)]
+        for acct in self._accounts.values():
+            for p in acct.pages:
+                seen[p] += 1
         for p in range(self.num_pages):
-            if counts[p] != self._refs[p]:
-                raise AssertionError(f"page {p}: {counts[p]} holders but reference count {self._refs[p]}")
-            if (p in free) != (self._refs[p] == 0):
-                raise AssertionError(f"page {p}: free list and reference count disagree")
-        if self.available_pages < 0:
-            raise AssertionError("more pages promised than free")
+            if seen[p] != self._holders[p]:
+                raise AssertionError(f"page {p} has {seen[p]} holders but a count of {self._holders[p]}")
+            if (p in free) == bool(seen[p]):
+                raise AssertionError(f"page {p} is {'free and held' if seen[p] else 'neither free nor held'}")
+        if self._promised != sum(a.promised for a in self._accounts.values()) or self.n_unpromised < 0:
+            raise AssertionError("the promises do not add up")
 
-    def _decref(self, page: int) -> None:
-        self._refs[page] -= 1
-        if self._refs[page] < 0:
-            raise RuntimeError(f"page {page} freed twice")
-        if self._refs[page] == 0:
-            heapq.heappush(self._free, page)
+    # -- internals -----------------------------------------------------------------------
+    def _account(self, owner: int) -> _Account:
+        try:
+            return self._accounts[owner]
+        except KeyError:
+            raise KeyError(f"owner {owner} has no account") from None
 
-    def _check_id(self, page: int) -> None:
+    def _valid(self, page: int) -> int:
         if not 0 <= page < self.num_pages:
-            raise IndexError(f"page {page} outside [0, {self.num_pages})")
+            raise IndexError(f"page {page} is outside [0, {self.num_pages})")
+        return page
+
+    def _let_go(self, page: int) -> None:
+        count = self._holders[page] - 1
+        if count < 0:
+            raise RuntimeError(f"page {page} was given back more often than it was taken")
+        self._holders[page] = count
+        if count == 0:
+            heapq.heappush(self._returned, page)

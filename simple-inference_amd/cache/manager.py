@@ -7,7 +7,10 @@ Within a group every run of a layer that writes keys and values has one *slab* o
 the pool, and one page id addresses that page in all slabs.
 
     keys    [slabs, pages + 1, kv_heads, page_size, head_dim]
-    values  [slabs, pages + 1, kv_heads, head_dim, page_size]
+    values  [slabs, pages + 1, kv_heads, value_dim, page_size]
+
+(``value_dim`` is ``head_dim`` unless the group's need says otherwise: a mixer may cache
+rows of another width beside its keys.)
 
 Values are stored with the positions innermost, so that the product
 ``probabilities x values`` reads consecutive positions as the matrix cores want
@@ -20,7 +23,7 @@ below ``s - window + 1`` go back to the allocator, and their table entries
 become -1.
 
 Beside the pages there are *slots*: one row of fixed size per running request
-and per stateful run of a layer, zeroed when a request gets its slot.  The
+and per stateful run of a layer, set to the state's initial value when a request gets its slot.  The
 architecture served here has no such state; the slots still exist, every request
 holds one, and the step function hands the slot ids to every mixer.
 """
@@ -34,7 +37,7 @@ import torch
 from ..parts.context import LayerCache
 from ..parts.model import CacheLayout
 from ..parts.plan import PagedKVNeed
-from .allocator import PageAllocator
+from .allocator import PagePool
 
 _STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
 
@@ -53,7 +56,7 @@ class PagedGroup:
         self.page_size = page_size
         self.num_pages = num_pages
         self.scratch_page = num_pages
-        self.allocator = PageAllocator(num_pages)
+        self.pool = PagePool(num_pages)
         self.tables: Dict[int, List[int]] = {}
         # a request's entry changes whenever its table does (graph replay skips rows that did not change); the
         # numbers come from one counter, so an id that is admitted again never meets a number it had before
@@ -62,7 +65,7 @@ class PagedGroup:
         self.k = self.v = None
         if allocate_storage:
             shape_k = (slabs, num_pages + 1, need.num_kv_heads, page_size, need.head_dim)
-            shape_v = (slabs, num_pages + 1, need.num_kv_heads, need.head_dim, page_size)
+            shape_v = (slabs, num_pages + 1, need.num_kv_heads, need.value_dim, page_size)
             self.k = torch.zeros(shape_k, dtype=dtype, device=device)
             self.v = torch.zeros(shape_v, dtype=dtype, device=device)
 
@@ -77,7 +80,7 @@ class PagedGroup:
         return min(full, pages_for(span, self.page_size) + 1)
 
     def begin(self, req: int, reserve: int) -> None:
-        self.allocator.reserve(req, reserve)
+        self.pool.open(req, reserve)
         self.tables[req] = []
         self._touch(req)
 
@@ -88,11 +91,11 @@ class PagedGroup:
             first_visible = max(0, start - self.need.window + 1)
             for idx in range(min(first_visible // self.page_size, len(table))):
                 if table[idx] >= 0:
-                    self.allocator.free_page(req, table[idx], back_to_reservation=True)
+                    self.pool.drop(req, table[idx], restore_promise=True)
                     table[idx] = -1
                     self._touch(req)
         while len(table) < pages_for(end, self.page_size):
-            table.append(self.allocator.allocate(req))
+            table.append(self.pool.take(req))
             self._touch(req)
 
     def _touch(self, req: int) -> None:
@@ -100,7 +103,7 @@ class PagedGroup:
         self.versions[req] = self._version
 
     def release(self, req: int) -> None:
-        self.allocator.release(req)
+        self.pool.close(req)
         self.tables.pop(req, None)
         self.versions.pop(req, None)
 
@@ -114,10 +117,11 @@ class StateSlots:
         self._free = list(range(max_running))
         self.slot_of: Dict[int, int] = {}
         self.tensors: List[Optional[torch.Tensor]] = []
+        self.initial = [need.init for need in states]
         for need in states:
             if allocate_storage:
-                self.tensors.append(torch.zeros((max_running + 1, *need.shape),
-                                                dtype=_STATE_DTYPES[need.dtype], device=device))
+                self.tensors.append(torch.full((max_running + 1, *need.shape), need.init,
+                                               dtype=_STATE_DTYPES[need.dtype], device=device))
             else:
                 self.tensors.append(None)
 
@@ -132,9 +136,9 @@ class StateSlots:
             raise MemoryError("no free state slot")
         slot = self._free.pop(0)  # lowest first (reference: ``serving/scheduler.py:59,116``)
         self.slot_of[req] = slot
-        for t in self.tensors:
+        for t, init in zip(self.tensors, self.initial):
             if t is not None:
-                t[slot].zero_()
+                t[slot].fill_(init)
         return slot
 
     def give_back(self, req: int) -> None:
@@ -164,7 +168,7 @@ class CacheManager:
         if total_tokens is None:
             return True
         return all(
-            g.pages_to_reserve(total_tokens, max_chunk) - shared_pages <= g.allocator.available_pages
+            g.pages_to_reserve(total_tokens, max_chunk) - shared_pages <= g.pool.n_unpromised
             for g in self.groups)
 
     def admit(self, req: int, total_tokens: Optional[int] = None, max_chunk: int = 1,
@@ -187,7 +191,7 @@ class CacheManager:
             reserve = 0 if total_tokens is None else max(0, g.pages_to_reserve(total_tokens, max_chunk) - len(shared))
             g.begin(req, reserve)
             for page in shared:
-                g.allocator.share(req, page)
+                g.pool.adopt(req, page)
                 g.tables[req].append(page)
                 g._touch(req)
         self.lengths[req] = len(shared) * self.page_size
@@ -200,6 +204,14 @@ class CacheManager:
             g.extend(req, start, start + new_tokens)
         self.lengths[req] = start + new_tokens
         return start
+
+    def retract(self, req: int, tokens: int) -> None:
+        """Takes back the last ``extend`` of a step that did not run after all.  Only the length goes back: the
+        pages stay the request's (the next ``extend`` finds them in its table), and pages that a window had
+        passed stay given back, since no later step could have seen them either."""
+        if not 0 <= tokens <= self.lengths[req]:
+            raise ValueError(f"request {req} holds {self.lengths[req]} tokens and cannot go back {tokens}")
+        self.lengths[req] -= tokens
 
     def release(self, req: int) -> None:
         for g in self.groups:
@@ -240,16 +252,16 @@ class CacheManager:
 
     # -- checks ------------------------------------------------------------
     def free_pages(self, group: int = 0) -> int:
-        return self.groups[group].allocator.free_pages
+        return self.groups[group].pool.n_free
 
     def check(self) -> None:
         for g in self.groups:
-            g.allocator.check()
+            g.pool.audit()
             for req, table in g.tables.items():
                 live = [p for p in table if p >= 0]
                 if len(set(live)) != len(live):
                     raise AssertionError(f"request {req} holds a page twice")
-                if set(live) != g.allocator.pages_of(req):
+                if set(live) != g.pool.pages(req):
                     raise AssertionError(f"request {req}: table and allocator disagree")
         slots = list(self.slots.slot_of.values())
         if len(set(slots)) != len(slots):

@@ -1,28 +1,40 @@
-"""Reuse of the pages of equal prompt prefixes (reference: ``serving/radix_cache.py:30-194``).
+"""Reuse of the pages of equal prompt prefixes (what the reference's ``serving/radix_cache.py:30-194`` is for).
 
-A tree keyed by complete pages of token ids; each node pins one page (all slabs of it) through an
-owner of its own in the page allocator, so a request that shares a prefix takes the pages by
-reference and nothing is copied.  A match covers complete pages only and leaves at least one
-prompt token to run (``((len - 1) // page) * page``), because the first new token needs logits.
-Least recently used leaves are dropped when admission needs their pages or the cache outgrows
-``max_pages``; a page stays alive while any request still holds it.
+A prompt's complete pages form a chain: page ``i`` is identified by its own token ids together with
+the identity of page ``i - 1``.  The cache is a flat table from ``(previous entry, token ids of a page)``
+to an entry that pins one page of the pool (all slabs of it), so a request with an equal prefix takes
+those pages by reference and nothing is copied.  A lookup covers complete pages only and always leaves
+at least one prompt token to run, because the first new token needs logits.
 
-It needs a model whose layers all keep every key (one group, no window) and that has no
-per-request state: a shared page must hold everything a later request needs of the prefix.
+What is dropped when admission needs pages, or when the cache outgrows ``capacity``, is the entry that
+ends a chain (nothing continues it) and was used longest ago.  Such entries wait in a heap ordered by
+their last use; the heap is cleaned lazily (an item is believed only if its entry still exists, still
+ends a chain and has not been used since), so a lookup, an insertion and an eviction each cost a few
+heap operations however many pages are cached.  A dropped page stays alive while a request still
+holds it.
+
+It needs a model whose layers all keep every key (one group, no window) and that has no per-request
+state: a shared page must hold everything a later request needs of the prefix.
 """
 
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Set, Tuple
+import heapq
+from typing import Dict, Iterable, List, Optional, Tuple
+
+_ROOT = 0
 
 
-class _Node:
-    __slots__ = ("key", "page", "owner", "parent", "children", "last_used")
+class _Entry:
+    __slots__ = ("uid", "page", "before", "edge", "continued_by", "used")
 
-    def __init__(self, key=None, page=None, owner=None, parent=None):
-        self.key, self.page, self.owner, self.parent = key, page, owner, parent
-        self.children: Dict[Tuple[int, ...], "_Node"] = {}
-        self.last_used = 0
+    def __init__(self, uid, page, before, edge, used):
+        self.uid = uid                  # identity of the chain up to and including this page
+        self.page = page
+        self.before = before            # the entry of the page in front (None for a prompt's first page)
+        self.edge = edge                # this entry's key in the table
+        self.continued_by = 0           # entries that have this one in front of them
+        self.used = used                # time of the last lookup or insertion that passed through
 
 
 class PrefixCache:
@@ -31,101 +43,120 @@ class PrefixCache:
             raise ValueError(f"max_pages must be positive, got {max_pages}")
         if len(cache.groups) != 1 or cache.groups[0].need.window is not None or cache.layout.states:
             raise ValueError("prefix reuse needs one cache group without a window and no per-request state")
-        self.cache = cache
-        self.allocator = cache.groups[0].allocator
+        self.pool = cache.groups[0].pool
         self.page_size = cache.page_size
-        self.max_pages = max_pages
-        self.root = _Node()
-        self.cached_pages = 0
-        self.hits = self.misses = self.matched_tokens = self.evictions = 0
-        self._clock = 0
-        self._next_owner = -1
+        self.capacity = max_pages
+        self._table: Dict[Tuple[int, Tuple[int, ...]], _Entry] = {}
+        self._ends: List[Tuple[int, int]] = []     # heap of (last use, uid) of entries that may end a chain
+        self._by_uid: Dict[int, _Entry] = {}
+        self._uids = _ROOT
+        self._now = 0
+        self.counters = {"lookups": 0, "lookups_hit": 0, "tokens_reused": 0, "pages_dropped": 0}
 
-    def _touch(self, node: _Node) -> None:
-        self._clock += 1
-        node.last_used = self._clock
+    def __len__(self) -> int:
+        return len(self._table)
+
+    # -- the two ways in -----------------------------------------------------------------
+    def _pages_of(self, tokens, n_tokens: int) -> Iterable[Tuple[int, ...]]:
+        ps = self.page_size
+        return (tuple(tokens[i:i + ps]) for i in range(0, n_tokens - ps + 1, ps))
+
+    def _use(self, entry: _Entry) -> None:
+        entry.used = self._now
+        if not entry.continued_by:
+            heapq.heappush(self._ends, (entry.used, entry.uid))
+            if len(self._ends) > 4 * len(self._table) + 64:    # mostly stale items: start the heap afresh
+                self._ends = [(e.used, e.uid) for e in self._table.values() if not e.continued_by]
+                heapq.heapify(self._ends)
 
     def match(self, tokens) -> List[int]:
-        """Pages of the longest cached prefix of ``tokens`` (complete pages, at least one token left over)."""
-        ps = self.page_size
-        reusable = ((len(tokens) - 1) // ps) * ps
-        node, pages = self.root, []
-        for start in range(0, reusable, ps):
-            child = node.children.get(tuple(tokens[start:start + ps]))
-            if child is None:
+        """Pages of the longest cached chain that starts ``tokens``, at least one token left over."""
+        self._now += 1
+        self.counters["lookups"] += 1
+        usable = (len(tokens) - 1) // self.page_size * self.page_size
+        found: List[int] = []
+        uid = _ROOT
+        for ids in self._pages_of(tokens, usable):
+            entry = self._table.get((uid, ids))
+            if entry is None:
                 break
-            self._touch(child)
-            pages.append(child.page)
-            node = child
-        if pages:
-            self.hits += 1
-            self.matched_tokens += len(pages) * ps
-        else:
-            self.misses += 1
-        return pages
+            self._use(entry)
+            found.append(entry.page)
+            uid = entry.uid
+        if found:
+            self.counters["lookups_hit"] += 1
+            self.counters["tokens_reused"] += len(found) * self.page_size
+        return found
 
     def insert(self, tokens, page_table: List[int]) -> None:
-        """Pins every complete page of a prompt whose keys and values are written."""
-        ps = self.page_size
-        complete = len(tokens) // ps
-        if len(page_table) < complete:
-            raise ValueError(f"prompt has {complete} complete pages but the table holds {len(page_table)}")
-        node = self.root
-        for i in range(complete):
-            key = tuple(tokens[i * ps:(i + 1) * ps])
-            child = node.children.get(key)
-            if child is None:
-                owner = self._next_owner
-                self._next_owner -= 1
-                self.allocator.reserve(owner, 0)
-                try:
-                    self.allocator.share(owner, page_table[i])
-                except Exception:
-                    self.allocator.release(owner)
-                    raise
-                child = _Node(key, page_table[i], owner, node)
-                node.children[key] = child
-                self.cached_pages += 1
-            self._touch(child)
-            node = child
-        while self.cached_pages > self.max_pages:
-            if not self._evict_one(set()):
-                break
+        """Keeps every complete page of ``tokens`` whose keys and values are written; ``page_table[i]`` is the
+        pool's page of positions ``i * page_size`` onwards."""
+        self._now += 1
+        whole = len(tokens) // self.page_size
+        if len(page_table) < whole:
+            raise ValueError(f"{whole} complete pages of tokens, but a table of {len(page_table)} pages")
+        before: Optional[_Entry] = None
+        for i, ids in enumerate(self._pages_of(tokens, whole * self.page_size)):
+            edge = (before.uid if before else _ROOT, ids)
+            entry = self._table.get(edge)
+            if entry is None:
+                self.pool.pin(page_table[i])      # raises for a page that nobody holds: nothing is recorded then
+                self._uids += 1
+                entry = _Entry(self._uids, page_table[i], before, edge, self._now)
+                self._table[edge] = self._by_uid[entry.uid] = entry
+                if before is not None:
+                    before.continued_by += 1
+            self._use(entry)
+            before = entry
+        while len(self._table) > self.capacity and self._drop_oldest_end(()):
+            pass
 
-    def evict_until_available(self, required_pages: int, protected: Optional[Set[int]] = None) -> bool:
-        protected = protected or set()
-        while self.allocator.available_pages < required_pages:
-            if not self._evict_one(protected):
+    # -- the way out ---------------------------------------------------------------------
+    def evict_until_available(self, required_pages: int, protected=()) -> bool:
+        """Drops chain ends, oldest first and never a ``protected`` page, until the pool has ``required_pages``
+        unpromised pages; False if it cannot get there."""
+        protected = frozenset(protected)
+        while self.pool.n_unpromised < required_pages:
+            if not self._drop_oldest_end(protected):
                 return False
         return True
 
-    def _nodes(self) -> List[_Node]:
-        out, stack = [], list(self.root.children.values())
-        while stack:
-            n = stack.pop()
-            out.append(n)
-            stack.extend(n.children.values())
-        return out
-
-    def _evict_one(self, protected: Set[int]) -> bool:
-        leaves = [n for n in self._nodes() if not n.children and n.page not in protected]
-        if not leaves:
+    def _drop_oldest_end(self, protected) -> bool:
+        spared = []
+        victim = None
+        while self._ends:
+            used, uid = heapq.heappop(self._ends)
+            entry = self._by_uid.get(uid)
+            if entry is None or entry.continued_by or entry.used != used:
+                continue                          # stale: dropped, continued or used again since
+            if entry.page in protected:
+                spared.append((used, uid))
+                continue
+            victim = entry
+            break
+        for item in spared:
+            heapq.heappush(self._ends, item)
+        if victim is None:
             return False
-        victim = min(leaves, key=lambda n: n.last_used)
-        del victim.parent.children[victim.key]
-        self.allocator.release(victim.owner)
-        self.cached_pages -= 1
-        self.evictions += 1
+        self._forget(victim)
+        self.counters["pages_dropped"] += 1
+        if victim.before is not None:
+            victim.before.continued_by -= 1
+            if not victim.before.continued_by:    # it ends a chain now, with the age it has
+                heapq.heappush(self._ends, (victim.before.used, victim.before.uid))
         return True
 
+    def _forget(self, entry: _Entry) -> None:
+        del self._table[entry.edge]
+        del self._by_uid[entry.uid]
+        self.pool.unpin(entry.page)
+
     def clear(self) -> None:
-        for n in self._nodes():
-            self.allocator.release(n.owner)
-        self.root.children.clear()
-        self.cached_pages = 0
-        self.hits = self.misses = self.matched_tokens = self.evictions = 0
+        for entry in list(self._table.values()):
+            self._forget(entry)
+        self._ends.clear()
+        for key in self.counters:
+            self.counters[key] = 0
 
     def stats(self) -> Dict[str, int]:
-        return {"cached_blocks": self.cached_pages, "cached_tokens": self.cached_pages * self.page_size,
-                "hits": self.hits, "misses": self.misses, "matched_tokens": self.matched_tokens,
-                "evictions": self.evictions}
+        return {"pages": len(self._table), "tokens": len(self._table) * self.page_size, **self.counters}

@@ -41,6 +41,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="do not launch a step before the tokens of the step before have been read")
     ap.add_argument("--use-prefix-cache", action="store_true")
+    ap.add_argument("--profile-ranges", action="store_true",
+                    help="named ranges around schedule / forward / sample / collect for a profiler's timeline")
     ap.add_argument("--stats-json", metavar="FILE", help="write the run's metrics there")
     ap.add_argument("--device", default="cuda:0")
     return ap
@@ -71,7 +73,8 @@ def main(argv=None) -> int:
     ecfg = EngineConfig(
         max_running=args.max_running, max_seq_len=args.max_seq_len, block_size=args.block_size,
         num_kv_blocks=args.num_kv_blocks, chunk_tokens=args.chunk_tokens, dtype=args.dtype,
-        use_graphs=not args.no_graphs, run_ahead=not args.no_run_ahead, use_prefix_cache=args.use_prefix_cache, device=args.device)
+        use_graphs=not args.no_graphs, run_ahead=not args.no_run_ahead, use_prefix_cache=args.use_prefix_cache, profile_ranges=args.profile_ranges,
+        device=args.device)
     print("Loading model...", file=sys.stderr, flush=True)
     if args.model:
         engine = Engine.from_folder(args.model, ecfg)

@@ -5,8 +5,9 @@ The names and meanings follow the keyword arguments of the reference's
 ``max_running``, ``max_seq_len``, ``block_size``, ``num_kv_blocks``,
 ``token_budget``, ``eos_id``, ``warmup``, ``use_prefix_cache`` and
 ``prefix_cache_blocks`` mean what they mean there; ``use_graphs`` is its
-``use_cuda_graphs`` (hipGraph here).  ``chunk_tokens``, ``dtype`` and ``run_ahead``
-have no counterpart there: the reference prefills whole prompts (``plan.md:811-868``
+``use_cuda_graphs`` (hipGraph here).  ``profile_ranges`` switches on the named
+ranges that the reference always records (``serving/engine.py:334,342,359``).  ``chunk_tokens``, ``dtype``
+and ``run_ahead`` have no counterpart there: the reference prefills whole prompts (``plan.md:811-868``
 only sketches portions) and has no 32-bit GPU path.
 """
 
@@ -49,6 +50,7 @@ class EngineConfig:
     use_prefix_cache: bool = False        # reuse complete pages of equal prompt prefixes
     prefix_cache_blocks: Optional[int] = None
     warmup: bool = False
+    profile_ranges: bool = False          # named ranges (profiler, roctx) around schedule / forward / sample / collect
     device: str = "cuda:0"
 
     def __post_init__(self):

@@ -26,11 +26,15 @@
 // probabilities are rounded to bfloat16 for the value product (reference:
 // kernels/attention_kernel.py:184-251 does the same in its prefill kernel).
 //
-// decode:  n_splits workgroups of four waves per (kv head, sequence); the sequence's tiles are dealt evenly, in
-//          order, to these waves (runs differ by a tile at most, whatever the length); the query heads that
-//          share the kv head are the q columns (at most 16).  A workgroup's four partial results are merged
-//          through LDS; (m, l, acc) per split go to a workspace and a second kernel combines the splits in
-//          order (a single split writes its result itself).
+// decode:  workgroups of four waves; a (kv head, sequence) is shared by as many of them ("splits") as its own
+//          number of visible key tiles says (decode_splits below: a power of two that leaves a wave some four
+//          tiles), never by how many sequences the step holds or how long the others are: the grid is sized for
+//          the longest sequence the step may hold, and workgroups beyond a sequence's own count leave at once.
+//          The sequence's tiles are dealt evenly, in order, to these waves (runs differ by a tile at most); the
+//          query heads that share the kv head are the q columns (at most 16).  A workgroup's four partial results
+//          are merged through LDS; (m, l, acc) per split go to a workspace and a second kernel combines the
+//          splits in order (a sequence with a single split writes its result itself).  So a sequence's result
+//          depends on its own keys and length only, bit for bit, whatever else is in the batch.
 // prefill: 128 consecutive tokens of one query head a workgroup (64 for head sizes over 128), as 4 waves of 32
 //          tokens or 8 waves of 16; the waves share each tile of keys and values through LDS (two stages;
 //          head sizes whose stages fit 64 KiB, the others load operands straight from the pages).
@@ -274,6 +278,17 @@ __device__ __forceinline__ void load_q(bf16x8 (&q)[KSTEPS], const bf16_t* row, i
 // decode: sequences with one new token each
 // ---------------------------------------------------------------------------------------------------
 constexpr int DEC_WAVES = 4;
+constexpr int DEC_TILES_PER_SPLIT = 16;  // a split is worth taking from this many tiles (512 keys) on
+constexpr int DEC_MAX_SPLITS = 32;
+
+// Workgroups that share one (sequence, kv head) with n_tiles visible key tiles: the largest power of two that
+// leaves every workgroup DEC_TILES_PER_SPLIT tiles, at most DEC_MAX_SPLITS.  A function of the sequence's own
+// length only; host and device use the same one.
+__host__ __device__ inline int decode_splits(int n_tiles) {
+    int s = 1;
+    while (s < DEC_MAX_SPLITS && 2 * s * DEC_TILES_PER_SPLIT <= n_tiles) s *= 2;
+    return s;
+}
 
 __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
@@ -281,21 +296,22 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const int* __restrict__ kv_len, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
     bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window) {
     extern __shared__ float lds[];  // [DEC_WAVES][group][HD + 2]
-    const int split = blockIdx.x, n_splits = gridDim.x, hk = blockIdx.y, seq = blockIdx.z;
+    // splits are the slowest index of the grid: the workgroups that leave at once (splits a sequence does not
+    // have) then come last, not interleaved with the others, which the chip deals out to its dies in turn
+    const int hk = blockIdx.x, seq = blockIdx.y, split = blockIdx.z, max_splits = gridDim.z;
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
-    scale *= LOG2E;  // exponentials are taken as powers of two
-    const int group = n_heads / n_kv;
-    const int* table = block_table + (size_t)seq * table_width;
-    // The queries do not depend on the sequence's length: they are loaded beside it (sequence s's one token
-    // is row s of the batch).
-    bf16x8 qf[1][KSTEPS];
-    load_q(qf[0], r < group ? q + (size_t)seq * q_row_stride + (hk * group + r) * HD : nullptr, g);
-
     // The tiles that hold visible keys are dealt evenly, in order, to the n_splits * DEC_WAVES waves that
     // work for this (sequence, kv head): every wave gets a contiguous run, runs differ by one tile at most.
     const int pos = kv_len[seq] - 1;
     const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
     const int t_first = lo_all / TILE, n_tiles = pos / TILE - t_first + 1;
+    const int n_splits = min(decode_splits(n_tiles), max_splits);
+    if (split >= n_splits) return;  // the whole workgroup: the grid is sized for the longest sequence there may be
+    scale *= LOG2E;  // exponentials are taken as powers of two
+    const int group = n_heads / n_kv;
+    const int* table = block_table + (size_t)seq * table_width;
+    bf16x8 qf[1][KSTEPS];
+    load_q(qf[0], r < group ? q + (size_t)seq * q_row_stride + (hk * group + r) * HD : nullptr, g);
     const int n_waves = n_splits * DEC_WAVES, wi = split * DEC_WAVES + wave;
     const int my_first = t_first + (int)(((long long)wi * n_tiles) / n_waves);
     const int my_end = t_first + (int)(((long long)(wi + 1) * n_tiles) / n_waves);
@@ -342,7 +358,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
             out[((size_t)cu_q[seq] * n_heads + hk * group + c) * HD + d] = float_to_bf16(o * (1.f / lsum));
             continue;
         }
-        const size_t slot = ((size_t)seq * n_heads + hk * group + c) * n_splits + split;
+        const size_t slot = ((size_t)seq * n_heads + hk * group + c) * max_splits + split;
         ws_acc[slot * HD + d] = o;
         if (d == 0) {
             ws_ml[slot * 2] = mx;
@@ -356,10 +372,14 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
 // 0), summed in split order, eight splits' loads in flight at a time.
 __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
     const float* __restrict__ ws_acc, const float* __restrict__ ws_ml, const int* __restrict__ cu_q,
-    bf16_t* __restrict__ out, int n_heads, int n_splits) {
+    const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int max_splits, int window) {
     const int head = blockIdx.x, seq = blockIdx.y, lane = threadIdx.x;
+    const int pos = kv_len[seq] - 1;
+    const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
+    const int n_splits = min(decode_splits(pos / TILE - lo_all / TILE + 1), max_splits);
+    if (n_splits == 1) return;  // its one workgroup wrote the result itself
     const int first = 0, last = n_splits - 1;
-    const size_t base = ((size_t)seq * n_heads + head) * n_splits;
+    const size_t base = ((size_t)seq * n_heads + head) * max_splits;
     float mx = -INFINITY;
     for (int s0 = first; s0 <= last; s0 += SIA_WAVE) {
         const int s = s0 + lane;
@@ -709,27 +729,40 @@ static int log2_exact(int v) {
 
 SIA_EXPORT int sia_attn_mfma_head_dim() { return HD; }
 
-// Sequences 0 .. n_seqs-1 of the step, each with exactly one new token, which is row s of q (cu_q[s] = s).
-// n_splits workgroups share the keys of each (sequence, kv head); ws_acc holds n_seqs * n_heads * n_splits *
-// head_dim floats, ws_ml n_seqs * n_heads * n_splits * 2.
+// Most workgroups that share one (sequence, kv head) when no sequence of the step holds more than kv_bound keys
+// (with a window: sees more than the window): what the caller sizes the workspaces and this library its grid by.
+SIA_EXPORT int sia_attn_decode_max_splits(int kv_bound, int window) {
+    if (kv_bound <= 0) return 1;
+    // the visible keys of a sequence of length n span at most this many tiles (a window need not start on a tile)
+    const int tiles_all = (kv_bound + TILE - 1) / TILE;
+    const int tiles = window > 0 ? min(tiles_all, (window + TILE - 2) / TILE + 1) : tiles_all;
+    return decode_splits(tiles);
+}
+
+// Sequences 0 .. n_seqs-1 of the step, each with exactly one new token, which is row s of q (cu_q[s] = s), and
+// none longer than kv_bound.  max_splits = sia_attn_decode_max_splits(kv_bound, window); ws_acc holds n_seqs *
+// n_heads * max_splits * head_dim floats, ws_ml n_seqs * n_heads * max_splits * 2 (neither is read before it is
+// written).
 SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                                const int* block_table, int table_width, const int* cu_q, const int* kv_len,
                                void* out, float* ws_acc, float* ws_ml, int n_seqs, int n_heads, int n_kv,
-                               int page_size, float scale, int window, int n_splits, hipStream_t stream) {
+                               int page_size, float scale, int window, int max_splits, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     const int ps_log2 = log2_exact(page_size);
-    if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || n_splits <= 0 || n_splits > 65535 ||
-        n_kv > 65535 || n_seqs > 65535 || q_row_stride % 8 || table_width <= 0)
+    const int n_splits = max_splits;
+    if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || n_splits <= 0 ||
+        n_splits > DEC_MAX_SPLITS || n_kv > 65535 || n_seqs > 65535 || q_row_stride % 8 || table_width <= 0 ||
+        (n_splits > 1 && (!ws_acc || !ws_ml)))
         return SIA_BAD_ARGUMENT;
     const size_t lds_bytes = (size_t)DEC_WAVES * (n_heads / n_kv) * (HD + 2) * sizeof(float);
     if (lds_bytes > 64 * 1024) return SIA_BAD_ARGUMENT;
-    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_splits, n_kv, n_seqs), dim3(DEC_WAVES * SIA_WAVE), lds_bytes,
+    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_kv, n_seqs, n_splits), dim3(DEC_WAVES * SIA_WAVE), lds_bytes,
                        stream, (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
                        block_table, table_width, cu_q, kv_len, ws_acc, ws_ml, (bf16_t*)out, n_heads, n_kv, ps_log2,
                        scale, window);
     if (n_splits > 1)
         hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_heads, n_seqs), dim3(SIA_WAVE), 0, stream, ws_acc,
-                           ws_ml, cu_q, (bf16_t*)out, n_heads, n_splits);
+                           ws_ml, cu_q, kv_len, (bf16_t*)out, n_heads, n_splits, window);
     return SIA_LAUNCH_CHECK();
 }
 

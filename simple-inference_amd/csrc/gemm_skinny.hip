@@ -2,9 +2,12 @@
 // the matrix products of a decode step, where every weight is read once and the time is the time
 // to stream W from HBM.
 //
-// One workgroup of 8 or 16 waves per 16*RB rows of W.  The waves split K between them in interleaved
-// chunks, so that the workgroup walks its rows front to back; their partial sums are added through
-// LDS in wave order.  A wave's step covers 64 k of RB blocks of 16 rows with 2*RB MFMAs 16x16x32:
+// One workgroup of 8 or 16 waves per 16*RB rows of W.  K is cut into chunks of 128, and chunk c belongs to
+// *share* c % 16: a share's chunks are summed front to back into one accumulator, and the 16 shares' sums are
+// added as (s0 + s8) + (s1 + s9) + ... + (s7 + s15), left to right.  With 16 waves every wave has one share
+// and the sums meet in LDS; with 8, wave w has shares w and w + 8 (chunks w, w + 8, w + 16, ... alternate
+// between its two accumulators) and adds the two itself, so the workgroup still walks its rows front to back
+// and needs half the LDS.  A wave's step covers 64 k of RB blocks of 16 rows with 2*RB MFMAs 16x16x32:
 //   A = W[n0 + 16 rb + r][k0 + 16g .. + 15]   two 16-byte loads a lane, 128 contiguous bytes per row
 //   B = X[r][same k]                           (rows r >= M are zero), loaded once for all RB blocks
 // (an MFMA's k index only has to mean the same element in A and B, so lane group g may take the 16
@@ -12,14 +15,17 @@
 // caches, once per workgroup: a workgroup takes as many row blocks (4, 2 or 1) as still leave some 160
 // workgroups, which is what measurements of the decode shapes favour.
 //
-// The result element (m, n) is summed over k in an order that depends on N and K only: a row's
-// result does not depend on M or on the other rows.
+// The result element (m, n) is summed over k in an order that depends on K only, not on M, the other rows,
+// the number of waves, the row blocks of a workgroup or the depth of its pipeline: whichever shape a launch
+// takes, a row's result is the same bit for bit.
 #include "common.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-constexpr int SK_STEP = 64;  // k per step of one wave
+constexpr int SK_STEP = 64;    // k per step of one wave
+constexpr int SK_CHUNK = 128;  // k per chunk: two steps
+constexpr int SK_SHARES = 16;  // chunk c is summed into share c % 16
 
 __device__ __forceinline__ bf16x8 ld8(const bf16_t* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
@@ -60,8 +66,8 @@ struct Epilogue {
     RowScale scale;
 };
 
-// RB: blocks of 16 rows of W per workgroup; WAVES: waves that split K; UNROLL: steps whose loads are in flight
-// together.
+// RB: blocks of 16 rows of W per workgroup; WAVES: 8 or 16 waves that split K; DEPTH: chunks (of two steps) whose
+// loads a wave has in flight together.
 //   EPI_STORE:   row block rb holds rows n0 + 16 rb ..: Y[m][n0 + 16 rb + n]  (TOut)
 //   EPI_SWIGLU:  W = [gate; up] of N rows each; the first RB / 2 row blocks are gate rows n0 + 16 j .., the others
 //                the up rows of the same columns: Y[m][n0 + 16 j + n] = silu(gate) * up, in float, rounded once
@@ -73,15 +79,16 @@ struct Epilogue {
 //                RMSNorm(x) W^T = rsqrt(mean x^2 + eps) * ((x * gain) W^T): the kernel leaves x * gain and the sums
 //                of squares of its own 16-column blocks, and the product after it (SCALED) adds those up, in an
 //                order that depends on N only, and scales its rows: no kernel of its own for the norm.
-template <typename TOut, int RB, int WAVES, int UNROLL, int EPI, bool SCALED>
+template <typename TOut, int RB, int WAVES, int DEPTH, int EPI, bool SCALED>
 __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                      const bf16_t* __restrict__ W,
                                                                      TOut* __restrict__ Y, int M, int N, int K,
                                                                      const Epilogue ep) {
+    static_assert(WAVES == 8 || WAVES == 16, "8 or 16 waves share the 16 shares of K");
+    constexpr int SPW = SK_SHARES / WAVES;  // shares per wave
     __shared__ float part[WAVES][RB][16][17];
-    __shared__ float squares[WAVES][16];
+    __shared__ float squares[SK_SHARES][16];
     const RopeOut& rope = ep.rope;
-    constexpr int CHUNK = SK_STEP * UNROLL;  // one wave's share of a round
     constexpr int OUT_BLOCKS = EPI == EPI_SWIGLU ? RB / 2 : RB;  // 16-column blocks of Y per workgroup
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int rope_half = EPI == EPI_ROPE ? rope.head_dim / 2 : 0;
@@ -100,16 +107,19 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
         w_row[rb] = W + (size_t)row * K + g * 16;
     }
 
-    // requested before the weights, used after them
-    constexpr int SQ_LANES = WAVES * 4;  // threads per row that add up the sums of squares
-    const int sq_m = lane & 15, sq_l = wave * 4 + (lane >> 4);
-    float sq[4] = {0.f, 0.f, 0.f, 0.f};
+    // requested before the weights, used after them.  The sums of squares of a row are added up the way the
+    // products are: 64 runners (16 shares of 4 lane groups), runner l taking partials l, l + 64, ...
+    constexpr int SQ_RUNNERS = SK_SHARES * 4;
+    const int sq_m = lane & 15;
+    float sq[SPW][4];
     if (SCALED) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int p = sq_l + i * SQ_LANES;
-            if (p < ep.scale.n_partials) sq[i] = ep.scale.partials[p * 16 + sq_m];
-        }
+        for (int j = 0; j < SPW; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int p = (wave + j * WAVES) * 4 + (lane >> 4) + i * SQ_RUNNERS;
+                sq[j][i] = p < ep.scale.n_partials ? ep.scale.partials[p * 16 + sq_m] : 0.f;
+            }
     }
     constexpr int RES_ITER = (RB * 256 + WAVES * SIA_WAVE - 1) / (WAVES * SIA_WAVE);
     float res_old[RES_ITER], res_gain[RES_ITER];
@@ -124,42 +134,67 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
         }
     }
 
-    floatx4 acc[RB];
+    // acc[j] belongs to share wave + j * WAVES; this wave's t-th chunk is chunk wave + t * WAVES, of share
+    // (wave + t * WAVES) % 16 = wave + (t % SPW) * WAVES: its accumulator t % SPW.
+    floatx4 acc[SPW][RB];
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) acc[rb] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = wave * CHUNK; k0 < K; k0 += WAVES * CHUNK) {
-        bf16x8 a[UNROLL][RB][2], b[UNROLL][2];
+    for (int j = 0; j < SPW; ++j)
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int k = k0 + u * SK_STEP;
-            const bool in = k < K;  // K is a multiple of 64: a step is inside or outside as a whole
+        for (int rb = 0; rb < RB; ++rb) acc[j][rb] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // A trip takes SPW * DEPTH of the wave's chunks: for each of its shares in turn, DEPTH chunks of that share
+    // are loaded together and then multiplied, front to back.
+    for (int k0 = wave * SK_CHUNK; k0 < K; k0 += SPW * DEPTH * WAVES * SK_CHUNK) {
 #pragma unroll
-            for (int rb = 0; rb < RB; ++rb) {
-                a[u][rb][0] = in ? ld8(w_row[rb] + k) : zero;
-                a[u][rb][1] = in ? ld8(w_row[rb] + k + 8) : zero;
-            }
-            b[u][0] = (in && x_live) ? ld8(x_row + k) : zero;
-            b[u][1] = (in && x_live) ? ld8(x_row + k + 8) : zero;
+        for (int j = 0; j < SPW; ++j) {
+            bf16x8 a[DEPTH][2][RB][2], b[DEPTH][2][2];
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int k = k0 + (d * SPW + j) * WAVES * SK_CHUNK + u * SK_STEP;
+                    const bool in = k < K;  // K is a multiple of 64: a step is inside or outside as a whole
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb) {
+                        a[d][u][rb][0] = in ? ld8(w_row[rb] + k) : zero;
+                        a[d][u][rb][1] = in ? ld8(w_row[rb] + k + 8) : zero;
+                    }
+                    b[d][u][0] = (in && x_live) ? ld8(x_row + k) : zero;
+                    b[d][u][1] = (in && x_live) ? ld8(x_row + k + 8) : zero;
+                }
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb) {
+                        acc[j][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[d][u][rb][0], b[d][u][0], acc[j][rb], 0, 0, 0);
+                        acc[j][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[d][u][rb][1], b[d][u][1], acc[j][rb], 0, 0, 0);
+                    }
         }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u)
-#pragma unroll
-            for (int rb = 0; rb < RB; ++rb) {
-                acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][rb][0], b[u][0], acc[rb], 0, 0, 0);
-                acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][rb][1], b[u][1], acc[rb], 0, 0, 0);
-            }
     }
-    // acc[rb][i] = partial of row m = r, column 4g + i of row block rb
+    // acc[j][rb][i] = share wave + j * WAVES of row m = r, column 4g + i of row block rb
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) part[wave][rb][r][g * 4 + i] = acc[rb][i];
+        for (int i = 0; i < 4; ++i)
+            part[wave][rb][r][g * 4 + i] = SPW == 2 ? acc[0][rb][i] + acc[SPW - 1][rb][i] : acc[0][rb][i];
+    // the sum over all of k of element (j, m, n): pairs of shares s and s + 8, then the pairs left to right
+    auto total = [&](int j, int m, int n) -> float {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) s += WAVES == 16 ? part[w][j][m][n] + part[w + 8][j][m][n] : part[w][j][m][n];
+        return s;
+    };
     if (SCALED) {
-        float ss = (sq[0] + sq[1]) + (sq[2] + sq[3]);
-        for (int p = sq_l + 4 * SQ_LANES; p < ep.scale.n_partials; p += SQ_LANES) ss += ep.scale.partials[p * 16 + sq_m];
-        ss += __shfl_xor(ss, 16);
-        ss += __shfl_xor(ss, 32);
-        if (lane < 16) squares[wave][lane] = ss;
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) {
+            float ss = (sq[j][0] + sq[j][1]) + (sq[j][2] + sq[j][3]);
+            for (int p = (wave + j * WAVES) * 4 + (lane >> 4) + 4 * SQ_RUNNERS; p < ep.scale.n_partials; p += SQ_RUNNERS)
+                ss += ep.scale.partials[p * 16 + sq_m];
+            ss += __shfl_xor(ss, 16);
+            ss += __shfl_xor(ss, 32);
+            if (lane < 16) squares[wave + j * WAVES][lane] = ss;
+        }
     }
     __syncthreads();
     // the row's scale: every thread that finishes an element of row m adds the waves' sums in the same order
@@ -167,18 +202,13 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
         if (!SCALED) return 1.f;
         float ss = 0.f;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) ss += squares[w][m];
+        for (int w = 0; w < SK_SHARES; ++w) ss += squares[w][m];
         return rsqrtf(ss / (float)K + ep.scale.eps);
     };
     if (EPI == EPI_ROPE) {
         const int m = threadIdx.x / 16, n = threadIdx.x % 16;
         if (threadIdx.x >= 256 || m >= M) return;
-        float a = 0.f, b = 0.f;  // columns j and j + half of the head
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w) {
-            a += part[w][0][m][n];
-            b += part[w][1][m][n];
-        }
+        float a = total(0, m, n), b = total(1, m, n);  // columns j and j + half of the head
         const float rs = row_scale(m);
         a *= rs;
         b *= rs;
@@ -218,9 +248,7 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
             const int idx = threadIdx.x + it * WAVES * SIA_WAVE;
             const int j = idx / 256, m = (idx / 16) % 16, n = idx % 16;
             if (idx >= RB * 256 || m >= M) continue;  // a whole 16-lane group leaves or stays
-            float s = 0.f;
-#pragma unroll
-            for (int w = 0; w < WAVES; ++w) s += part[w][j][m][n];
+            const float s = total(j, m, n);
             const float x = res_old[it] + bf16_to_float(float_to_bf16(s * row_scale(m)));
             const size_t at = (size_t)m * N + n0 + j * 16 + n;
             ep.res.residual[at] = x;
@@ -239,20 +267,12 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
         if (m >= M) continue;
         const float rs = row_scale(m);
         if (EPI == EPI_SWIGLU) {
-            float gate = 0.f, up = 0.f;
-#pragma unroll
-            for (int w = 0; w < WAVES; ++w) {
-                gate += part[w][j][m][n];
-                up += part[w][OUT_BLOCKS + j][m][n];
-            }
+            float gate = total(j, m, n), up = total(OUT_BLOCKS + j, m, n);
             gate *= rs;
             up *= rs;
             Y[(size_t)m * N + n0 + j * 16 + n] = from_float<TOut>(gate / (1.f + expf(-gate)) * up);
         } else {
-            float s = 0.f;
-#pragma unroll
-            for (int w = 0; w < WAVES; ++w) s += part[w][j][m][n];
-            Y[(size_t)m * N + n0 + j * 16 + n] = from_float<TOut>(s * rs);
+            Y[(size_t)m * N + n0 + j * 16 + n] = from_float<TOut>(total(j, m, n) * rs);
         }
     }
 }
@@ -264,17 +284,17 @@ SIA_EXPORT int sia_gemm_skinny_max_rows() { return 16; }
 template <typename TOut, int EPI>
 static void launch_skinny(const bf16_t* X, const bf16_t* W, TOut* Y, int M, int N, int K, const Epilogue& ep,
                           hipStream_t stream) {
-#define LAUNCH(RB, WAVES, UNROLL)                                                                                \
-    hipLaunchKernelGGL((gemm_skinny_kernel<TOut, RB, WAVES, UNROLL, EPI, false>), dim3(N / (16 * RB)),             \
+#define LAUNCH(RB, WAVES, DEPTH)                                                                                 \
+    hipLaunchKernelGGL((gemm_skinny_kernel<TOut, RB, WAVES, DEPTH, EPI, false>), dim3(N / (16 * RB)),              \
                        dim3(WAVES * SIA_WAVE), 0, stream, X, W, Y, M, N, K, ep)
     if (N % 64 == 0 && N / 64 >= 160)
-        LAUNCH(4, 8, 2);
+        LAUNCH(4, 8, 1);
     else if (N % 32 == 0 && N / 32 >= 160 && K >= 1024)
-        LAUNCH(2, 16, 2);
+        LAUNCH(2, 16, 1);
     else if (M <= 4)
-        LAUNCH(1, 8, 4);
-    else
         LAUNCH(1, 8, 2);
+    else
+        LAUNCH(1, 8, 1);
 #undef LAUNCH
 }
 
@@ -314,7 +334,7 @@ SIA_EXPORT int sia_gemm_skinny_swiglu(const void* X, const void* W, void* Y, int
     ep.scale = RowScale{partials, n_partials, eps};
     const bool wide = inter % 32 == 0 && inter / 32 >= 160 && K >= 1024 && M > 4;
 #define LAUNCH(RB, WAVES, SCALED)                                                                                  \
-    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, RB, WAVES, 2, EPI_SWIGLU, SCALED>), dim3(inter / (8 * RB)),      \
+    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, RB, WAVES, 1, EPI_SWIGLU, SCALED>), dim3(inter / (8 * RB)),      \
                        dim3(WAVES * SIA_WAVE), 0, stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, inter, \
                        K, ep)
     if (wide && partials)
@@ -350,7 +370,7 @@ SIA_EXPORT int sia_gemm_skinny_rope(const void* X, const void* W, void* Y, int M
     ep.scale = RowScale{partials, n_partials, eps};
     const dim3 grid(heads * (head_dim / 32));
 #define LAUNCH(WAVES, SCALED)                                                                                      \
-    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 2, WAVES, 2, EPI_ROPE, SCALED>), grid, dim3(WAVES * SIA_WAVE), 0, \
+    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 2, WAVES, 1, EPI_ROPE, SCALED>), grid, dim3(WAVES * SIA_WAVE), 0, \
                        stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K, ep)
     if (K >= 1024 && partials)
         LAUNCH(16, true);

@@ -19,6 +19,7 @@ one token too far; that token is dropped, and its slot goes to the next request 
 
 from __future__ import annotations
 
+import sys
 import time
 from typing import Dict, Iterator, List, Optional, Sequence
 
@@ -29,8 +30,10 @@ from ..config.engine_config import EngineConfig
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .build import default_kernels, model_from_folder, model_from_random
+from .ranges import NamedRanges
 from .request import Request, RequestState
 from .scheduler import Scheduler
+from .graphs import GraphedDecode, GraphUnavailable
 from .step import StepEntry, StepRunner
 
 
@@ -63,9 +66,10 @@ class Engine:
             self.prefix_cache = PrefixCache(self.cache, max_pages=cap)
         self.graphs = None
         if engine_cfg.graphs_wanted():
-            from .graphs import GraphedDecode
             self.graphs = GraphedDecode(self)
-        self.stats = {"steps": 0, "tokens_run": 0, "prefill_tokens": 0, "decode_tokens": 0, "steps_ahead": 0}
+        self.stats = {"steps": 0, "tokens_run": 0, "prefill_tokens": 0, "decode_tokens": 0, "steps_ahead": 0,
+                      "graph_fallbacks": 0}
+        self.ranges = NamedRanges(engine_cfg.profile_ranges)
         self._ahead = None   # a step launched but not yet read: (requests that sampled a token, those tokens)
         self._token_mirrors = None   # two pinned host buffers that sampled tokens are copied into, in turn
         self._mirror_turn = 0
@@ -110,17 +114,16 @@ class Engine:
         vocab = self.model.vocab_size
         if any(t < 0 or t >= vocab for t in prompt):
             raise ValueError("prompt contains out-of-range token ids")
-        req = Request(prompt_tokens=prompt, params=params)
-        self.scheduler.add(req)
+        req = Request(prompt, params)
+        self.scheduler.submit(req)
         return req
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work() or self._ahead is not None
+        return self.scheduler.busy() or self._ahead is not None
 
     def reset(self) -> None:
         """Drops every request and gives every page and slot back."""
-        self.scheduler.waiting.clear()
-        self.scheduler.running.clear()
+        self.scheduler.clear()
         self._ahead = None
         self.cache.reset()
         if self.prefix_cache is not None:
@@ -128,20 +131,20 @@ class Engine:
 
     # -- admission ----------------------------------------------------------------
     def _try_admit(self, req: Request) -> bool:
-        total = req.prompt_len + req.max_new_tokens
+        """The scheduler's gate: finds the request a slot and the pages of its whole length (those of an equal
+        prefix by reference) and lets it enter, or says no."""
         shared: List[int] = []
         if self.prefix_cache is not None:
             shared = self.prefix_cache.match(req.prompt_tokens)
             if self._prefix_still_being_written(req, len(shared)):
                 return False
-            need = self.cache.groups[0].pages_to_reserve(total, self.cfg.chunk_tokens) - len(shared)
-            if not self.prefix_cache.evict_until_available(need, protected=set(shared)):
+            need = self.cache.groups[0].pages_to_reserve(req.total_len, self.cfg.chunk_tokens) - len(shared)
+            if not self.prefix_cache.evict_until_available(need, protected=shared):
                 return False
-        if not self.cache.can_admit(total, self.cfg.chunk_tokens, len(shared)):
+        if not self.cache.can_admit(req.total_len, self.cfg.chunk_tokens, len(shared)):
             return False
-        req.slot = self.cache.admit(req.id, total, self.cfg.chunk_tokens, shared_pages=shared)
-        req.cached_prefix_len = len(shared) * self.cfg.block_size
-        req.num_computed = req.cached_prefix_len
+        slot = self.cache.admit(req.id, req.total_len, self.cfg.chunk_tokens, shared_pages=shared)
+        req.enter(slot, reused_tokens=len(shared) * self.cfg.block_size)
         return True
 
     def _prefix_still_being_written(self, req: Request, matched_pages: int) -> bool:
@@ -152,7 +155,7 @@ class Engine:
         reusable = (req.prompt_len - 1) // ps
         if matched_pages >= reusable:
             return False
-        for other in self.scheduler.running:
+        for other in self.scheduler.live:
             if other.state is not RequestState.PREFILL:
                 continue
             limit = min(reusable, other.prompt_len // ps)
@@ -182,48 +185,56 @@ class Engine:
         """Plans a step and puts it on the GPU.  ``before``: the step launched before it whose tokens the host has
         not read (its decoding requests take their input from its sampled tokens on the device), or None.
         Returns (requests that sample a token, their tokens), or None if there is nothing to run."""
-        self.scheduler.evict_finished()
-        plan = self.scheduler.plan_step(self._try_admit)   # admits, too: into steps with room for prompt tokens
+        with self.ranges("engine.schedule"):
+            self.scheduler.retire()      # their pages and slots went back when they finished
+            plan = self.scheduler.plan(self._try_admit)   # lets requests in, too: into steps with room for their tokens
         if not plan:
             return None
         entries, emitters = [], []
         for req, n in plan:
-            if req.state is RequestState.DECODE:
-                if req.pending:    # its input is still on the device
-                    entries.append(StepEntry(req.id, [0], [0], token_from=req.pending_row))
-                else:
-                    entries.append(StepEntry(req.id, [req.last_token], [0]))
+            kind = "decode_tokens" if req.state is RequestState.DECODE else "prefill_tokens"
+            tokens, samples, device_row = req.take(n)
+            entries.append(StepEntry(req.id, tokens, [n - 1] if samples else [], token_from=device_row))
+            if samples:
                 emitters.append(req)
-                self.stats["decode_tokens"] += 1
-            else:
-                tokens = req.prompt_tokens[req.num_computed:req.num_computed + n]
-                last = req.num_computed + n == req.prompt_len
-                entries.append(StepEntry(req.id, tokens, [n - 1] if last else []))
-                if last:
-                    emitters.append(req)
-                self.stats["prefill_tokens"] += n
+            self.stats[kind] += n
+            self.stats["tokens_run"] += n
         self.stats["steps"] += 1
         self.stats["steps_ahead"] += before is not None
-        self.stats["tokens_run"] += sum(n for _, n in plan)
 
         device_tokens = before[1][0] if before is not None and before[1] is not None else None
-        if self.graphs is not None and self.graphs.can_run(plan):
-            logits = self.graphs.run(entries, device_tokens)
-        else:
-            logits = self.runner.run(entries, device_tokens)
-        for req, n in plan:
-            req.num_computed += n
-            if self.prefix_cache is not None and req.state is RequestState.PREFILL:
-                # pages a prompt has filled so far can be shared from the next step on
-                self.prefix_cache.insert(req.prompt_tokens[:req.num_computed], self.cache.table(0, req.id))
+        with self.ranges("engine.forward"):
+            logits = self._forward(entries, device_tokens)
+        if self.prefix_cache is not None:
+            for req, _ in plan:
+                if req.state is RequestState.PREFILL:
+                    # pages a prompt has filled so far can be shared from the next step on
+                    self.prefix_cache.insert(req.prompt_tokens[:req.num_computed], self.cache.table(0, req.id))
         if not emitters:
             return [], None
-        tokens = self._sample(logits, emitters, [r.num_generated + r.pending for r in emitters])
+        with self.ranges("engine.sample"):
+            tokens = self._sample(logits, emitters, [r.num_generated + r.in_flight for r in emitters])
         for row, req in enumerate(emitters):
-            req.state = RequestState.DECODE   # a prompt that has just ended decodes from the next step on
-            req.pending += 1
-            req.pending_row = row
+            req.sampled(row)
         return emitters, tokens
+
+    def _forward(self, entries: List[StepEntry], device_tokens):
+        """One call of the step function: a replayed graph where the step is one token for every request, else
+        eager.  A graph that cannot be captured or replayed is given up for good (reference:
+        ``serving/engine.py:300-309,478-497``): the same entries run eagerly, on the books as they were."""
+        if self.graphs is not None and self.graphs.can_run(entries):
+            try:
+                return self.graphs.run(entries, device_tokens)
+            except GraphUnavailable as exc:
+                self._give_up_graphs(exc)
+        return self.runner.run(entries, device_tokens)
+
+    def _give_up_graphs(self, exc) -> None:
+        cause = exc.__cause__ or exc
+        print(f"[engine] graph replay failed ({type(cause).__name__}: {cause}); decode steps run eagerly from here on",
+              file=sys.stderr, flush=True)
+        self.graphs = None
+        self.stats["graph_fallbacks"] += 1
 
     def _sample(self, logits, emitters: List[Request], draw_indices: List[int]):
         """Samples on the device and starts the copy of the tokens to the host right behind the sampler, so that
@@ -248,43 +259,32 @@ class Engine:
         return tokens, read
 
     def _collect(self, emitters: List[Request], tokens) -> Dict[int, int]:
-        """Reads a launched step's sampled tokens and books them."""
+        """Reads a launched step's sampled tokens and books them.  A request that ends gives its pages and slot
+        back at once: the next step may hand them out.  One that had ended on an end-of-sequence token a step ago
+        (this step ran ahead of that news) drops its token."""
         emitted: Dict[int, int] = {}
         if not emitters:
             return emitted
-        for req, token in zip(emitters, tokens[1]()):
-            req.pending -= 1
-            if req.state is RequestState.FINISHED:
-                continue   # ended on an end-of-sequence token a step ago; this step ran ahead of that news
-            self._emit(req, int(token))
-            emitted[req.id] = int(token)
+        with self.ranges("engine.collect"):
+            for req, token in zip(emitters, tokens[1]()):
+                if req.deliver(int(token), self.eos_ids):
+                    emitted[req.id] = int(token)
+                    if req.state is RequestState.FINISHED:
+                        self.cache.release(req.id)
         return emitted
 
     def _next_step_is_certain(self, emitters: List[Request]) -> bool:
         """True if the step after the one whose tokens are still on the device can be planned without them: none
         of its requests reaches ``max_new_tokens`` with the token it is about to get.  (An end-of-sequence token
         is found out a step late.)"""
-        return bool(self.cfg.run_ahead and emitters) and all(
-            r.num_generated + r.pending < r.max_new_tokens for r in emitters)
-
-    def _emit(self, req: Request, token: int) -> None:
-        """Appends a token and moves the request on (reference: ``serving/engine.py:449-460,499-507``)."""
-        req.generated.append(token)
-        if token in self.eos_ids and not req.params.ignore_eos:
-            req.eos_hit = True
-        if req.should_finish():
-            req.state = RequestState.FINISHED
-            self.cache.release(req.id)   # pages and slot go back at once; the next step may hand them out
-            req.slot = None
+        return bool(self.cfg.run_ahead and emitters) and all(r.length_is_certain_after_next_token() for r in emitters)
 
     def run(self) -> Dict[int, Request]:
         """Steps until every queued request has finished; returns them by id."""
-        seen: Dict[int, Request] = {r.id: r for r in self.scheduler.waiting}
-        seen.update({r.id: r for r in self.scheduler.running})
+        seen: Dict[int, Request] = {r.id: r for r in (*self.scheduler.queue, *self.scheduler.live)}
         while self.has_work():
             self.step()
-            for r in self.scheduler.running:
-                seen[r.id] = r
+            seen.update((r.id, r) for r in self.scheduler.live)
         return seen
 
     def warmup(self, num_seqs: int = 2, prompt_len: int = 8, decode_steps: int = 4) -> None:
@@ -300,7 +300,10 @@ class Engine:
             self.step()
             guard -= 1
         if self.graphs is not None:
-            self.graphs.capture_all()
+            try:
+                self.graphs.capture_all()
+            except GraphUnavailable as exc:
+                self._give_up_graphs(exc)
         if self.device.type == "cuda":
             torch.cuda.synchronize(self.device)
         self.reset()

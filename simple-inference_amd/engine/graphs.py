@@ -29,6 +29,11 @@ from ..parts.context import StepContext
 from .step import StepEntry
 
 
+class GraphUnavailable(RuntimeError):
+    """A decode graph could not be captured or replayed.  The step it was asked for has not run, and the cache
+    manager's books are as they were before the call: the caller can run the same entries eagerly."""
+
+
 def buckets_for(max_running: int) -> List[int]:
     """1, 2, 4, ... and ``max_running`` itself (reference: buckets(7) = [1, 2, 4, 7])."""
     out, b = [], 1
@@ -83,8 +88,11 @@ class GraphedDecode:
             raise RuntimeError("graph replay needs the GPU")
 
     # -- which steps ---------------------------------------------------------------
-    def can_run(self, plan) -> bool:
-        return 0 < len(plan) <= self.buckets[-1] and all(n == 1 for _, n in plan)
+    def can_run(self, entries: List[StepEntry]) -> bool:
+        """A step can be replayed if every request brings one token and wants its logits.  (A prompt's portion of
+        one token that is not its last brings one token too, but wants nothing: such a step runs eagerly.)"""
+        return 0 < len(entries) <= self.buckets[-1] and all(
+            len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
 
     def bucket_of(self, rows: int) -> int:
         return next(b for b in self.buckets if b >= rows)
@@ -198,26 +206,37 @@ class GraphedDecode:
         for kv_bound in (kv_bounds or self.kv_buckets[-1:]):
             for size in self.buckets:
                 if (size, kv_bound) not in self._made:
-                    self.capture(size, kv_bound)
+                    self._capture_or_give_up(size, kv_bound)
+
+    def _capture_or_give_up(self, size: int, kv_bound: int) -> _Bucket:
+        try:
+            return self.capture(size, kv_bound)
+        except Exception as exc:     # capture is fragile: memory for a private pool, a library that cannot be recorded
+            raise GraphUnavailable(f"capture of the graph for {size} rows and {kv_bound} positions failed") from exc
 
     @torch.no_grad()
     def run(self, entries: List[StepEntry], device_tokens=None) -> torch.Tensor:
         """Logits ``[len(entries), vocab]`` of a step of single tokens.  An entry with ``token_from`` holds a
         placeholder; its token id is that row of ``device_tokens`` (int32, on the device): the sampler's output of
-        the step before, which the host need not have read yet."""
+        the step before, which the host need not have read yet.  Raises ``GraphUnavailable``, with nothing
+        booked, if the graph cannot be captured or replayed."""
         self.runner._check(entries)
+        if not self.can_run(entries):
+            raise ValueError("a replayed step takes one token per request and returns its logits")
         for e in entries:
             if e.token_from is not None and (device_tokens is None or device_tokens.dtype != torch.int32
                                              or not 0 <= e.token_from < device_tokens.numel()):
                 raise ValueError("an entry takes its token from a row of int32 device_tokens that was not given")
-        for e in entries:
-            if len(e.tokens) != 1 or list(e.want) != [0]:
-                raise ValueError("a replayed step takes one token per request and returns its logits")
         size = self.bucket_of(len(entries))
         longest = max(self.cache.lengths[e.req] for e in entries) + 1
         kv_bound = self.kv_bucket_of(longest)
-        b = self._made.get((size, kv_bound)) or self.capture(size, kv_bound)
-        self._fill(b, entries, device_tokens)
-        b.graph.replay()
+        b = self._made.get((size, kv_bound)) or self._capture_or_give_up(size, kv_bound)
+        self._fill(b, entries, device_tokens)     # takes the step's pages: from here on the step is booked
+        try:
+            b.graph.replay()
+        except Exception as exc:
+            for e in entries:
+                self.cache.retract(e.req, 1)
+            raise GraphUnavailable(f"replay of the graph for {size} rows and {kv_bound} positions failed") from exc
         self.replays += 1
         return b.logits[:len(entries)]

@@ -1,23 +1,20 @@
-"""The scheduler: who is admitted, and which tokens of whom a step runs.
+"""The scheduler: who runs in the next step, with how many tokens, and who may come in.
 
-Admission is the reference's (``serving/scheduler.py:93-123``): first come first served; while
-there is a waiting request and a free slot, the head of the queue is admitted if the context
-already admitted plus its prompt fits ``token_budget`` (an idle engine always admits one) and if
-``can_admit`` (the cache manager promising its pages) says yes.  If the head cannot be admitted
-nobody behind it is: no overtaking.  Nothing is ever preempted: a request is promised the pages
-of its whole declared length before it starts, so pages cannot run out in mid-flight; when the
-pool is full the head of the queue waits until a finished request gives its pages back.
+One decision a step, ``plan``: every decoding request gets its one token, then the requests that are
+still on their prompts get portions, in the order they came in, until ``chunk_tokens`` tokens are in
+the step; into whatever room is left, requests are let in from the head of the queue and get their
+first portion at once.  So a request enters only in a step that can run some of its tokens: it does
+not hold a promise of pages while it could not run anyway, and prompts that arrive together are
+matched against the prefix cache after the earlier ones have written their pages.
 
-What the reference lacks is the cut of prompts into portions (``plan.md:811-868`` sketches it).
-``plan_step`` gives every decoding request its one token first, then hands prompt portions to
-the prefilling requests in admission order until ``chunk_tokens`` tokens are in the step.  A
-request turns to DECODE in the step that runs its last prompt token and emits its first token
-from that step.
-
-Given the admission test, ``plan_step`` also admits: a waiting request enters only in a step
-that still has room for its first prompt tokens.  So a request is not promised pages while it
-could not run anyway, and when prompts arrive together the later ones are matched against the
-prefix cache after the earlier ones have written their pages, not before.
+The rules of coming in are the reference's (``serving/scheduler.py:93-123``): first come first served;
+a free slot; the context already inside plus the newcomer's prompt within ``token_budget`` (an empty
+engine takes any one request); and the caller's ``gate`` (the cache manager promising its pages).  If
+the head of the queue cannot come in, nobody behind it does.  Nothing is ever put out again: a request
+is promised the pages of its whole declared length before it starts, so pages cannot run out in
+mid-flight; when the pool is full the head of the queue waits until a finished request gives its
+pages back.  The cut of prompts into portions has no counterpart in the reference (``plan.md:811-868``
+sketches it).
 """
 
 from __future__ import annotations
@@ -27,6 +24,8 @@ from typing import Callable, Deque, List, Optional, Tuple
 
 from .request import Request, RequestState
 
+Gate = Optional[Callable[[Request], bool]]
+
 
 class Scheduler:
     def __init__(self, max_running: int, token_budget: int, chunk_tokens: int):
@@ -35,73 +34,64 @@ class Scheduler:
         self.max_running = max_running
         self.token_budget = token_budget
         self.chunk_tokens = chunk_tokens
-        self.waiting: Deque[Request] = deque()
-        self.running: List[Request] = []
+        self.queue: Deque[Request] = deque()     # not yet let in, oldest first
+        self.live: List[Request] = []            # let in and not yet retired, in the order they came in
 
-    def add(self, req: Request) -> None:
-        req.state = RequestState.WAITING
-        self.waiting.append(req)
+    def submit(self, req: Request) -> None:
+        if req.state is not RequestState.WAITING:
+            raise ValueError(f"request {req.id} is {req.state.value}; only a waiting request can be queued")
+        self.queue.append(req)
 
-    def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+    def busy(self) -> bool:
+        return bool(self.queue) or bool(self.live)
 
-    def evict_finished(self) -> List[Request]:
-        done = [r for r in self.running if r.state is RequestState.FINISHED]
-        if done:
-            self.running = [r for r in self.running if r.state is not RequestState.FINISHED]
-        return done
+    def clear(self) -> None:
+        self.queue.clear()
+        self.live.clear()
 
-    def _running_tokens(self) -> int:
-        return sum(r.context_len for r in self.running)
+    def retire(self) -> List[Request]:
+        """Takes the finished requests out; returns them."""
+        gone = [r for r in self.live if r.state is RequestState.FINISHED]
+        if gone:
+            self.live = [r for r in self.live if r.state is not RequestState.FINISHED]
+        return gone
 
-    def admit(self, can_admit: Optional[Callable[[Request], bool]] = None,
-              limit: Optional[int] = None) -> List[Request]:
-        """Admits from the head of the queue while slots, the token budget and ``can_admit`` allow, at most
-        ``limit`` requests."""
-        admitted: List[Request] = []
-        used = self._running_tokens()
-        while self.waiting and len(self.running) < self.max_running and (limit is None or len(admitted) < limit):
-            head = self.waiting[0]
-            if (self.running or admitted) and used + head.prompt_len > self.token_budget:
-                break
-            if can_admit is not None and not can_admit(head):
-                break
-            self.waiting.popleft()
+    def let_in(self, gate: Gate = None) -> Optional[Request]:
+        """The head of the queue comes in if slot, budget and ``gate`` allow; returns it, or None.  ``gate`` is
+        expected to give the request its slot and pages (``Request.enter``); without one it just turns to PREFILL."""
+        if not self.queue or len(self.live) >= self.max_running:
+            return None
+        head = self.queue[0]
+        if self.live and sum(r.context_len for r in self.live) + head.prompt_len > self.token_budget:
+            return None
+        if gate is not None and not gate(head):
+            return None
+        self.queue.popleft()
+        if head.state is RequestState.WAITING:
             head.state = RequestState.PREFILL
-            self.running.append(head)
-            admitted.append(head)
-            used += head.prompt_len
-        return admitted
+        self.live.append(head)
+        return head
 
-    def plan_step(self, can_admit: Optional[Callable[[Request], bool]] = None,
-                  admit: bool = False) -> List[Tuple[Request, int]]:
-        """(request, number of its next tokens) for one step: decoded tokens, then prompt portions.
-
-        With ``admit`` (or an admission test), waiting requests are admitted one by one while the step
-        has room left for prompt tokens, and get their first portion in this step."""
-        plan: List[Tuple[Request, int]] = []
-        room = self.chunk_tokens
-        for r in self.running:
-            if r.state is RequestState.DECODE:
-                plan.append((r, 1))
-                room -= 1
-        for r in self.running:
+    def plan(self, gate: Gate = None, admit: bool = True) -> List[Tuple[Request, int]]:
+        """(request, number of its next tokens) for one step: decoded tokens first, then prompt portions, then the
+        first portions of requests that come in with this step (none with ``admit`` False)."""
+        step: List[Tuple[Request, int]] = [(r, 1) for r in self.live if r.state is RequestState.DECODE]
+        room = self.chunk_tokens - len(step)
+        for r in self.live:
+            if room <= 0:
+                break
             if r.state is RequestState.PREFILL:
-                if room <= 0:
-                    break
-                n = min(room, r.prompt_len - r.num_computed)
-                plan.append((r, n))
+                n = r.tokens_wanted(room)
+                step.append((r, n))
                 room -= n
-        if admit or can_admit is not None:
-            while room > 0:
-                newcomers = self.admit(can_admit, limit=1)
-                if not newcomers:
-                    break
-                r = newcomers[0]
-                n = min(room, r.prompt_len - r.num_computed)
-                plan.append((r, n))
-                room -= n
-        return plan
+        while admit and room > 0:
+            newcomer = self.let_in(gate)
+            if newcomer is None:
+                break
+            n = newcomer.tokens_wanted(room)
+            step.append((newcomer, n))
+            room -= n
+        return step
 
     def __repr__(self) -> str:
-        return f"Scheduler(waiting={len(self.waiting)}, running={len(self.running)}/{self.max_running})"
+        return f"<scheduler: {len(self.queue)} queued, {len(self.live)} of {self.max_running} slots live>"

@@ -54,6 +54,7 @@ _ATTN_SIGNATURES = {
                         _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_attn_prefill": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "sia_attn_decode_max_splits": [_c_int, _c_int],
     "sia_attn_prefill_rows": [],
     "sia_attn_prefill_rows_split": [],
     "sia_attn_prefill_rows_long": [],
@@ -248,8 +249,8 @@ class HipKernels:
         M, K = x.shape
         N = w.shape[0]
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
-            if (self.use_skinny_gemm and M <= self._skinny_rows and N % 16 == 0 and K % 64 == 0
-                    and (out_float32 or not (N < 4096 and K > 4096))):  # few long rows: the library is faster
+            # up to 16 rows: this package's kernel, whose sums do not depend on the number of rows
+            if self.use_skinny_gemm and M <= self._skinny_rows and N % 16 == 0 and K % 64 == 0:
                 y = torch.empty((M, N), dtype=torch.float32 if out_float32 else torch.bfloat16, device=x.device)
                 self._check(self.core.sia_gemm_skinny(_ptr(x), _ptr(w), _ptr(y), M, N, K, int(out_float32),
                                                       self._stream()), "gemm_skinny")
@@ -402,8 +403,7 @@ class HipKernels:
         k and v columns are not to be read (for few rows one kernel does all three and never writes them)."""
         M, K = x.shape
         if (self.use_skinny_gemm and self.fuse_rope and n_kv_written and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
-                and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 32 == 0 and K % 64 == 0
-                and not ((n_heads + 2 * n_kv_written) * head_dim < 4096 and K > 4096)):
+                and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 32 == 0 and K % 64 == 0):
             x, partials, n_partials, norm_eps = self._scaled(x)
             self._want(x, "q/k/v input")
             self._want(w_qkv, "q/k/v weight")
@@ -465,20 +465,6 @@ class HipKernels:
             self._stream()), "attention_generic")
         return out
 
-    @staticmethod
-    def decode_split(n_seqs: int, n_kv_heads: int, kv_bound: int) -> int:
-        """Number of workgroups (four waves each) that share the keys of one (sequence, kv head).  The
-        kernel deals a sequence's tiles of 32 keys evenly to the waves.  Splits are taken while they still give
-        every one of the 256 compute units at most one workgroup, in powers of two (which deal the tiles of the
-        usual lengths evenly), and no more than leave every wave about two tiles at the longest length the step
-        can hold.  Measured at 2,048 and 8,192 keys and 1 to 64 sequences: a split that puts a second workgroup
-        on some compute units, or an odd one, costs more than it gains (12 sequences of 8 kv heads: 2 splits
-        26 us, 3 splits 34 us; 24 sequences: 1 split 40 us, 2 splits 48 us)."""
-        fits = max(1, 256 // max(1, n_seqs * n_kv_heads))
-        most = max(1, kv_bound // (2 * 4 * 32))
-        want = min(fits, most)
-        return 1 << (want.bit_length() - 1)
-
     def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
         lib = self._attn_lib(head_dim)
         width = qkv.shape[1]
@@ -486,14 +472,17 @@ class HipKernels:
         group = n_heads // n_kv_heads
         n_dec = ctx.n_decode_seqs if group <= 16 and 4 * group * (head_dim + 2) * 4 <= 65536 else 0
         if n_dec:
-            bound = ctx.kv_bound or ctx.max_kv_len
-            n_splits = self.decode_split(n_dec, n_kv_heads, bound)
-            ws_acc = torch.empty((n_dec * n_heads * n_splits * head_dim,), dtype=torch.float32, device=qkv.device)
-            ws_ml = torch.empty((n_dec * n_heads * n_splits * 2,), dtype=torch.float32, device=qkv.device)
+            # How many workgroups share a (sequence, kv head) is the kernel's decision, from that sequence's own
+            # length; the step's longest possible sequence only sizes the grid and the workspaces.
+            max_splits = lib.sia_attn_decode_max_splits(int(ctx.kv_bound or ctx.max_kv_len), window)
+            ws_acc = ws_ml = None
+            if max_splits > 1:
+                ws_acc = torch.empty((n_dec * n_heads * max_splits * head_dim,), dtype=torch.float32, device=qkv.device)
+                ws_ml = torch.empty((n_dec * n_heads * max_splits * 2,), dtype=torch.float32, device=qkv.device)
             self._check(lib.sia_attn_decode(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), _ptr(ws_acc), _ptr(ws_ml), n_dec, n_heads,
-                n_kv_heads, cache.page_size, float(scale), window, n_splits, self._stream()),
+                n_kv_heads, cache.page_size, float(scale), window, max_splits, self._stream()),
                 "attn_decode")
         if n_dec < ctx.n_seqs:
             rows, rows_split = lib.sia_attn_prefill_rows(), lib.sia_attn_prefill_rows_split()

@@ -75,16 +75,28 @@ class TensorSpec:
 
 @dataclass(frozen=True)
 class PagedKVNeed:
-    """Keys and values in pages: all keys (``window`` None) or the last ``window``."""
+    """Keys and values in pages: all keys (``window`` None) or the last ``window``.
+
+    A page holds, per key/value head, ``page_size`` key rows of ``head_dim`` elements and as many value rows of
+    ``value_head_dim`` elements (None: the same width).  The cache manager only stores them; what a row means is
+    the mixer's affair, so a mixer that caches something narrower or wider beside its keys names that width here.
+    """
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_head_dim: Optional[int] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.value_head_dim is None else self.value_head_dim
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Per-request state of fixed size (one row per running request)."""
+    """Per-request state of fixed size (one row per running request).  A request's row holds ``init`` in every
+    element when the request gets its slot."""
 
     shape: Tuple[int, ...]
     dtype: str = "float32"
+    init: float = 0.0

@@ -4,61 +4,103 @@ import random
 
 import pytest
 
-from simple_inference_amd.cache import CacheManager, PageAllocator
+from simple_inference_amd.cache import CacheManager, PagePool
 from simple_inference_amd.parts.model import CacheLayout
 from simple_inference_amd.parts.plan import PagedKVNeed, StateNeed
 import torch
 
 
-def test_allocator_vector_of_the_reference_test():
+def test_pool_vector_of_the_reference_test():
     """serving/test_paged_kv_cache.py:27-43."""
-    a = PageAllocator(4)
-    a.reserve(1, 2)
-    a.reserve(2, 1)
-    assert not a.can_reserve(3, 2)
-    assert (a.allocate(1), a.allocate(1)) == (0, 1)
-    a.share(2, 0)
-    assert a.ref_count(0) == 2
-    a.release(1)
-    assert a.ref_count(0) == 1 and a.free_pages == 3
-    a.release(2)
-    assert a.free_pages == 4
-    a.check()
+    a = PagePool(4)
+    a.open(1, promise=2)
+    a.open(2, promise=1)
+    assert not a.fits(2) and a.fits(1)
+    assert (a.take(1), a.take(1)) == (0, 1)
+    a.adopt(2, 0)
+    assert a.holders(0) == 2
+    a.close(1)
+    assert a.holders(0) == 1 and a.n_free == 3
+    a.close(2)
+    assert a.n_free == 4
+    a.audit()
 
 
-def test_allocator_errors():
-    a = PageAllocator(2)
+def test_pool_errors():
+    a = PagePool(2)
     with pytest.raises(KeyError):
-        a.allocate(9)
-    a.reserve(1, 1)
+        a.take(9)
+    a.open(1, promise=1)
     with pytest.raises(ValueError):
-        a.can_reserve(1, 1)
+        a.open(1, promise=1)
     with pytest.raises(MemoryError):
-        a.reserve(2, 2)
-    p = a.allocate(1)
-    a.reserve(2, 1)
-    with pytest.raises(MemoryError):       # reservation used up and the other page is promised
-        a.allocate(1)
+        a.open(2, promise=2)
+    assert not a.has(2)
+    p = a.take(1)
+    a.open(2, promise=1)
+    with pytest.raises(MemoryError):       # promise used up and the other page is promised
+        a.take(1)
     with pytest.raises(ValueError):
-        a.share(1, p)
+        a.adopt(1, p)
     with pytest.raises(ValueError):
-        a.share(2, 1)                      # page 1 is free
-    a.free_page(1, p)
-    with pytest.raises(KeyError):          # freed twice
-        a.free_page(1, p)
-    a.release(1), a.release(2), a.release(77)
-    assert a.free_pages == 2
-    a.check()
+        a.adopt(2, 1)                      # page 1 is free
+    with pytest.raises(IndexError):
+        a.holders(2)
+    a.drop(1, p)
+    with pytest.raises(KeyError):          # given back twice
+        a.drop(1, p)
+    a.close(1), a.close(2), a.close(77)
+    assert a.n_free == 2
+    a.audit()
 
 
-def test_unreserved_allocation_takes_unpromised_pages_only():
-    a = PageAllocator(3)
-    a.reserve(1, 0)
-    a.reserve(2, 2)
-    assert a.allocate(1) == 0              # one page is promised to nobody
+def test_an_account_without_a_promise_takes_unpromised_pages_only():
+    a = PagePool(3)
+    a.open(1)
+    a.open(2, promise=2)
+    assert a.take(1) == 0                  # one page is promised to nobody
     with pytest.raises(MemoryError):
-        a.allocate(1)
-    assert (a.allocate(2), a.allocate(2)) == (1, 2)
+        a.take(1)
+    assert (a.take(2), a.take(2)) == (1, 2)
+
+
+def test_pages_come_back_lowest_first_from_below_and_above_the_watermark():
+    a = PagePool(6)
+    a.open(1)
+    got = [a.take(1) for _ in range(4)]
+    assert got == [0, 1, 2, 3]
+    a.drop(1, 2), a.drop(1, 0)
+    assert [a.take(1) for _ in range(3)] == [0, 2, 4]     # returned ids before ids never handed out
+    a.audit()
+
+
+def test_pins_keep_a_page_alive_outside_every_account():
+    a = PagePool(2)
+    a.open(1)
+    p = a.take(1)
+    a.pin(p), a.pin(p)
+    a.close(1)
+    assert a.n_free == 1 and a.holders(p) == 2
+    a.audit()
+    a.unpin(p)
+    assert a.n_free == 1
+    a.unpin(p)
+    assert a.n_free == 2
+    with pytest.raises(KeyError):
+        a.unpin(p)
+    with pytest.raises(ValueError):
+        a.pin(p)                           # a free page
+    a.audit()
+
+
+def test_a_dropped_page_can_become_a_promise_again():
+    a = PagePool(2)
+    a.open(1, promise=2)
+    p, q = a.take(1), a.take(1)
+    a.drop(1, p, restore_promise=True)
+    assert a.n_free == 1 and a.n_unpromised == 0 and not a.fits(1)
+    assert a.take(1) == p
+    a.audit()
 
 
 def layout(groups, slabs=None, states=()):
@@ -110,7 +152,7 @@ def test_reservation_makes_running_out_impossible_in_mid_flight():
     with pytest.raises(MemoryError):
         m.extend(1, 2)                     # beyond what it declared, and nothing is left
     m.release(1), m.release(2)
-    assert m.free_pages() == 4 and m.groups[0].allocator.reserved_pages == 0
+    assert m.free_pages() == 4 and m.groups[0].pool.n_promised == 0
 
 
 def test_window_group_gives_pages_back_when_the_window_has_passed():
@@ -155,8 +197,9 @@ def test_window_reservation_is_small_and_sufficient():
     m.check()
 
 
-def test_slots_lowest_first_zeroed_and_scratch():
-    m = manager([FULL], states=[StateNeed((2,), "float32")], storage=True, max_running=2)
+def test_slots_lowest_first_set_to_their_initial_value_and_scratch():
+    m = manager([FULL], states=[StateNeed((2,), "float32"), StateNeed((3,), "float32", init=-1.5)], storage=True,
+                max_running=2)
     s0, s1 = m.admit(10), m.admit(11)
     assert (s0, s1) == (0, 1) and m.slots.scratch_slot == 2
     state = m.slots.tensors[0]
@@ -166,7 +209,11 @@ def test_slots_lowest_first_zeroed_and_scratch():
     with pytest.raises(MemoryError):
         m.admit(12)
     m.release(10)
-    assert m.admit(13) == 0 and float(state[0].abs().sum()) == 0.0   # zeroed on assignment
+    other = m.slots.tensors[1]
+    assert other.shape == (3, 3) and bool((other == -1.5).all())
+    other[0] = 4.0
+    assert m.admit(13) == 0 and float(state[0].abs().sum()) == 0.0   # set anew on assignment
+    assert bool((other[0] == -1.5).all())
     m.check()
 
 
@@ -180,7 +227,7 @@ def test_shared_prefix_pages():
     m.extend(2, 2)
     assert m.table(0, 2)[:2] == first_two and m.table(0, 2)[2] not in m.table(0, 1)
     m.release(1)
-    assert m.groups[0].allocator.ref_count(first_two[0]) == 1   # still held by request 2
+    assert m.groups[0].pool.holders(first_two[0]) == 1   # still held by request 2
     m.release(2)
     assert m.free_pages() == 6
 
@@ -218,13 +265,13 @@ def test_random_orders_lose_no_page(seed):
             del live[r]
         m.check()
         for g in m.groups:
-            held = sum(len(g.allocator.pages_of(o)) for o in g.allocator.owners())
-            assert held + g.allocator.free_pages == g.num_pages
+            held = sum(len(g.pool.pages(o)) for o in g.pool.owners())
+            assert held + g.pool.n_free == g.num_pages
     for r in list(live):
         m.release(r)
     m.check()
     assert all(m.free_pages(g) == 40 for g in range(2)) and m.slots.free_slots == 4
-    assert all(g.allocator.reserved_pages == 0 for g in m.groups)
+    assert all(g.pool.n_promised == 0 for g in m.groups)
 
 
 def test_a_table_version_never_comes_back():

@@ -214,24 +214,18 @@ def test_running_a_step_ahead_changes_no_token(folders, name, dtype):
     for a slot all get the tokens they get without running ahead, sampled ones included, and every page comes
     back.  A request that has run past its end-of-sequence token keeps its row for one step, and a request that
     arrives while a step is running ahead joins one step later, so the rows of a step are then not the same in
-    the two runs; in bfloat16, where the choice of kernel by the number of rows shows in the last bits, no
-    request ends on a token here and all arrive before the first step."""
+    the two runs.  Decode steps do not mind (a row's result does not depend on the other rows, in either dtype);
+    a step with a prompt in it does in bfloat16, where its products, the decoding rows' too, go to the BLAS
+    library, which picks its method by the number of rows: there all requests arrive before the first step and
+    find a slot at once, so that every later step is a decode step."""
     tiny = TINIES[name]
     vocab = tiny.config["vocab_size"]
     prompts = [random_tokens(vocab, n, seed=80 + i) for i, n in enumerate((5, 23, 9, 31, 14, 3))]
     first_params = SamplingParams(max_new_tokens=12, temperature=1.0, seed=7)
-    probe = engine(folders[name], tiny, dtype, run_ahead=False, max_running=1)
-    first = probe.add_request(prompts[0], params=first_params)
-    probe.run()
-    first = first.generated
-    # request 0 ends on this token, in the middle of its allowance
-    stop = next((t for i, t in enumerate(first) if 3 <= i < 10 and t not in first[:i]), None)
-    assert stop is not None, first
-    if dtype == "bfloat16":
-        stop = -1
 
-    def stream(run_ahead):
-        eng = engine(folders[name], tiny, dtype, run_ahead=run_ahead, eos_id=stop, max_running=4)
+    def stream(run_ahead, stop):
+        eng = engine(folders[name], tiny, dtype, run_ahead=run_ahead, eos_id=stop,
+                     max_running=4 if dtype == "float32" else 6, chunk_tokens=24 if dtype == "float32" else 96)
         params = [first_params,
                   SamplingParams(max_new_tokens=20, temperature=0.8, top_k=20, top_p=0.9, seed=3),
                   SamplingParams(max_new_tokens=7, temperature=0.0, ignore_eos=True),
@@ -251,9 +245,160 @@ def test_running_a_step_ahead_changes_no_token(folders, name, dtype):
         assert eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks()
         return [r.generated for r in reqs], eng.stats["steps_ahead"]
 
-    plain_way, none_ahead = stream(False)
-    ahead_way, some_ahead = stream(True)
+    # request 0 ends on a token of its own, in the middle of its allowance: what it generates in this arrangement
+    # when no token stops it says which (in bfloat16 that need not be what it generates alone: its prompt shares
+    # its first step with others, and the products of such a step depend on the step's size)
+    first = stream(False, -1)[0][0]
+    stop = next((t for i, t in enumerate(first) if 3 <= i < 10 and t not in first[:i]), None)
+    assert stop is not None, first
+    plain_way, none_ahead = stream(False, stop)
+    ahead_way, some_ahead = stream(True, stop)
     assert none_ahead == 0 and some_ahead > 0
     assert plain_way == ahead_way
-    if stop >= 0:
-        assert plain_way[0][-1] == stop and 4 <= len(plain_way[0]) <= 10   # the end-of-sequence token ended request 0
+    assert plain_way[0][-1] == stop and 4 <= len(plain_way[0]) <= 10   # the end-of-sequence token ended request 0
+
+
+@pytest.mark.parametrize("chunk_tokens", [1, 4, 5])
+def test_portions_of_one_token_beside_decoders_with_graphs(folders, chunk_tokens):
+    """A step budget at or below the number of slots: prompts are then fed a token or two at a time, and a step in
+    which every request brings one token may hold a prompt's token that is not its last (nothing is sampled for
+    it).  Such a step is not a decode step and must not go to a replayed graph; every request still generates
+    what it generates alone."""
+    tiny = TINIES["b"]
+    vocab = tiny.config["vocab_size"]
+    prompts = [random_tokens(vocab, n, seed=160 + i) for i, n in enumerate((3, 10, 1, 7, 5, 9))]
+
+    def run(prompts_now, **kw):
+        eng = engine(folders["b"], tiny, "float32", **kw)
+        handles, waiting, steps = [], list(prompts_now), 0
+        while waiting or eng.has_work():
+            if waiting and steps % 3 == 0:          # arrivals while others decode
+                handles.append(eng.add_request(waiting.pop(0), max_new_tokens=6))
+            eng.step()
+            steps += 1
+            assert steps < 400
+        eng.cache.check()
+        assert eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks()
+        return [h.generated for h in handles], eng
+
+    alone = [run([p], max_running=1, use_graphs=False)[0][0] for p in prompts]
+    got, eng = run(prompts, max_running=4, chunk_tokens=chunk_tokens, use_graphs=True)
+    assert got == alone
+    assert eng.stats["graph_fallbacks"] == 0 and eng.graphs is not None
+    if chunk_tokens > 1:
+        assert eng.graphs.replays > 0
+
+
+@pytest.mark.parametrize("broken", ["capture", "replay"])
+def test_a_graph_that_cannot_be_captured_or_replayed_falls_back_to_eager_steps(folders, broken, monkeypatch, capfd):
+    """serving/engine.py:300-309,478-497 in kind: the failing call is made to raise from the host; the step runs
+    eagerly on the same books (no page taken twice, no position skipped) and every token is what it is without
+    graphs."""
+    from simple_inference_amd.engine.graphs import GraphedDecode
+    tiny = TINIES["d"]
+    vocab = tiny.config["vocab_size"]
+    prompts = [random_tokens(vocab, n, seed=170 + i) for i, n in enumerate((9, 30, 4))]
+    want = []
+    for dtype in ("float32",):
+        eager = engine(folders["d"], tiny, dtype, use_graphs=False)
+        reqs = [eager.add_request(p, max_new_tokens=10) for p in prompts]
+        eager.run()
+        want = [r.generated for r in reqs]
+    eng = engine(folders["d"], tiny, "float32", use_graphs=True)
+    calls = {"n": 0}
+    if broken == "capture":
+        def fail(self, size, kv_bound):
+            raise RuntimeError("no memory for the graph's private pool (made up by the test)")
+        monkeypatch.setattr(GraphedDecode, "capture", fail)
+    else:
+        real = GraphedDecode.capture
+
+        def capture_then_break(self, size, kv_bound):
+            bucket = real(self, size, kv_bound)
+
+            class Broken:
+                def replay(_):
+                    calls["n"] += 1
+                    if calls["n"] == 3:
+                        raise RuntimeError("replay refused (made up by the test)")
+                    bucket_graph.replay()
+            bucket_graph = bucket.graph
+            bucket.graph = Broken()
+            return bucket
+        monkeypatch.setattr(GraphedDecode, "capture", capture_then_break)
+    reqs = [eng.add_request(p, max_new_tokens=10) for p in prompts]
+    eng.run()
+    assert [r.generated for r in reqs] == want
+    assert eng.graphs is None and eng.stats["graph_fallbacks"] == 1
+    assert "decode steps run eagerly from here on" in capfd.readouterr().err
+    eng.cache.check()
+    assert eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks()
+
+
+@pytest.mark.parametrize("name", ["a", "d"])
+def test_decode_steps_in_bfloat16_do_not_depend_on_the_batch(folders, name):
+    """serving/test_engine.py:151-190 in the serving dtype.  Each request's prompt is run the same way in every
+    arrangement (alone, whole); then it decodes given tokens alone, among three others, among fifteen others, and
+    in replayed graphs padded to their bucket under a larger bound on the length: its logits are the same bit for
+    bit, because neither the few-row products nor the split of its keys between workgroups look at the rest of
+    the batch.  (A step of more than 16 rows sends its products to the BLAS library, which chooses its method by
+    the number of rows: such steps agree within rounding, see the test below.)"""
+    tiny = TINIES[name]
+    vocab = tiny.config["vocab_size"]
+    lengths = (5, 70, 33, 130, 1, 64, 17, 90, 12, 47, 8, 100, 3, 29, 55, 21)
+    prompts = [random_tokens(vocab, n, seed=180 + i) for i, n in enumerate(lengths)]
+    given = [random_tokens(vocab, 12, seed=220 + i) for i in range(len(prompts))]
+
+    def decode(groups, graphs):
+        """Logits [request][step] when the requests decode in the given groups (one batch a group and step)."""
+        eng = engine(folders[name], tiny, "bfloat16", use_graphs=graphs, max_running=16, max_seq_len=1024)
+        for i, p in enumerate(prompts):
+            eng.cache.admit(i)
+            eng.runner.run([StepEntry(i, p, [])])
+        out = {i: [] for i in range(len(prompts))}
+        for step in range(12):
+            for group in groups:
+                entries = [StepEntry(i, [given[i][step]], [0]) for i in group]
+                logits = eng.graphs.run(entries) if graphs else eng.runner.run(entries)
+                for row, i in enumerate(group):
+                    out[i].append(logits[row].clone())
+        return out
+
+    everyone = list(range(16))
+    alone = decode([[i] for i in everyone], graphs=False)
+    for groups, graphs in (([everyone[:4], everyone[4:7], everyone[7:]], False), ([everyone], False),
+                           ([everyone[:3], everyone[3:]], True), ([everyone[::-1]], True)):
+        got = decode(groups, graphs)
+        for i in everyone:
+            for step in range(12):
+                assert torch.equal(got[i][step], alone[i][step]), (groups, graphs, i, step)
+
+
+def test_random_request_streams_in_bfloat16_stay_within_rounding_of_the_plain_implementation(folders):
+    """The stream of the 32-bit test above in the serving dtype, greedy only.  Prompts are cut and batched as the
+    stream has it, so a request's steps differ from its steps alone in the number of rows of their products (the
+    BLAS library's choice from 17 rows on): its tokens need not be bit-equal to a solo run's, but every one of
+    them must be the plain implementation's choice, or tie with it within bfloat16 rounding."""
+    import random
+    folder, tiny = folders["b"], TINIES["b"]
+    V = tiny.config["vocab_size"]
+    rng = random.Random(11)
+    shared = [rng.randrange(V) for _ in range(40)]
+    reqs = []
+    for _ in range(14):
+        base = shared[:rng.randint(0, len(shared))] if rng.random() < 0.5 else []
+        reqs.append((base + [rng.randrange(V) for _ in range(rng.randint(1, 90))], rng.randint(1, 12)))
+    for kw in (dict(max_running=6, num_kv_blocks=60, chunk_tokens=32, use_graphs=True, use_prefix_cache=True),
+               dict(max_running=3, num_kv_blocks=40, chunk_tokens=16, use_graphs=True)):
+        eng = Engine.from_folder(folder, EngineConfig(dtype="bfloat16", max_seq_len=320, block_size=16, eos_id=-1, **kw))
+        handles, pending, step = [], list(reqs), 0
+        while pending or eng.has_work():
+            for _ in range(min(len(pending), random.Random(step).randint(0, 3))):
+                prompt, n = pending.pop(0)
+                handles.append(eng.add_request(prompt, max_new_tokens=n))
+            eng.step()
+            step += 1
+        eng.cache.check()
+        for (prompt, n), h in zip(reqs, handles):
+            assert len(h.generated) == n
+            greedy_matches_plain(folder, prompt, h.generated, "bfloat16")

@@ -384,6 +384,86 @@ def test_matrix_core_attention_decode_and_mixed(hip, geom):
         torch.testing.assert_close(plain_kernel.float(), ref.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("geom", [(24, 8, 128, 16, None), (6, 2, 48, 16, 700), (32, 8, 64, 64, None)])
+def test_decode_attention_of_a_sequence_does_not_depend_on_its_batch(hip, geom):
+    """How a sequence's keys are split between workgroups and merged follows from its own length: alone, beside
+    others, beside many, and under a larger bound on the length (as replayed graphs have it) its result is the
+    same bit for bit.  Lengths on both sides of every number of splits (1, 2, 4, 8, 16 from 512 keys a split)."""
+    n_heads, n_kv, D, ps, window = geom
+    dtype = torch.bfloat16
+    kv_lens = [1, 63, 511, 512, 1023, 1024, 1500, 2048, 2500, 4095, 4097, 9000]
+    pages = sum(-(-kv // ps) for kv in kv_lens) + 5
+    cache = Cache(pages, n_kv, ps, D, dtype, kv_lens, seed=8)
+    cache.k_pages.copy_(rnd(*cache.k_pages.shape, dtype=dtype, seed=9))
+    cache.v_pages.copy_(rnd(*cache.v_pages.shape, dtype=dtype, seed=10))
+    qkv = rnd(len(kv_lens), (n_heads + 2 * n_kv) * D, dtype=dtype, seed=11)
+    scale = 1 / math.sqrt(D)
+
+    def run(which, bound=0, repeat=1):
+        """Attention of the sequences ``which`` (each ``repeat`` times in the batch) as one decode step."""
+        ids = [i for i in which for _ in range(repeat)]
+        ctx = Ctx([1] * len(ids), [kv_lens[i] for i in ids])
+        ctx.kv_bound = bound
+        sub = Cache.__new__(Cache)
+        sub.page_size, sub.k_pages, sub.v_pages = ps, cache.k_pages, cache.v_pages
+        sub.block_table = cache.block_table[ids].contiguous()
+        out = hip.paged_attention(qkv[ids].contiguous(), n_heads, n_kv, D, scale, window, ctx, sub)
+        return {i: out[j * repeat] for j, i in enumerate(which)}
+
+    everyone = list(range(len(kv_lens)))
+    together = run(everyone)
+    ref = twin.paged_attention(qkv, n_heads, n_kv, D, scale, window, Ctx([1] * len(kv_lens), kv_lens), cache)
+    torch.testing.assert_close(torch.stack([together[i] for i in everyone]).float(), ref.float(), **tol(dtype))
+    bounded = run(everyone, bound=16384)
+    many = run(everyone, repeat=6)                    # 72 sequences: more workgroups than compute units
+    for i in everyone:
+        alone = run([i])[i]
+        assert torch.equal(alone, together[i]), kv_lens[i]
+        assert torch.equal(alone, bounded[i]), kv_lens[i]
+        assert torch.equal(alone, many[i]), kv_lens[i]
+    pair = run([3, 9])
+    assert torch.equal(pair[3], together[3]) and torch.equal(pair[9], together[9])
+
+
+def test_few_row_products_do_not_depend_on_the_number_of_rows(hip):
+    """Up to 16 rows every product (plain, gated, into the residual, with the norm's row scale, with rotation and
+    cache write) sums k in an order that K alone fixes: a row's result is the same bit for bit whether it runs
+    alone, among 4, among 5 (another kernel shape from 5 rows on) or among 16."""
+    from simple_inference_amd.kernels import ScaledRows
+    dtype = torch.bfloat16
+    for N, K in ((3072, 8192), (5120, 3072), (16384, 3072), (1008, 1024), (48, 192)):
+        x, w = rnd(16, K, dtype=dtype, seed=1), rnd(N, K, dtype=dtype, seed=2, scale=K ** -0.5)
+        full = hip.linear(x, w)
+        full32 = hip.linear(x, w, out_float32=True)
+        for m in (1, 4, 5, 11):
+            assert torch.equal(hip.linear(x[:m].contiguous(), w), full[:m]), (N, K, m)
+            assert torch.equal(hip.linear(x[:m].contiguous(), w, out_float32=True), full32[:m]), (N, K, m)
+            assert torch.equal(hip.linear(x[m - 1:m].contiguous(), w), full[m - 1:m]), (N, K, m)
+    for inter, K in ((8192, 3072), (96, 320), (5120, 1024)):
+        x = rnd(16, K, dtype=dtype, seed=3)
+        w = rnd(2 * inter, K, dtype=dtype, seed=4, scale=K ** -0.5)
+        full = hip.gated_linear(x, w)
+        for m in (1, 4, 5, 11):
+            assert torch.equal(hip.gated_linear(x[:m].contiguous(), w), full[:m]), (inter, K, m)
+    # into the residual, and out of it again through the row scale of the products that follow
+    hidden, inner, inter = 3072, 8192, 8192
+    x = rnd(16, inner, dtype=dtype, seed=5)
+    w = rnd(hidden, inner, dtype=dtype, seed=6, scale=inner ** -0.5)
+    w_gu = rnd(2 * inter, hidden, dtype=dtype, seed=7, scale=hidden ** -0.5)
+    res = rnd(16, hidden, seed=8, scale=2.0)
+    gain = (rnd(hidden, seed=9, scale=0.3) + 1.0).contiguous()
+
+    def through(m):
+        r = res[:m].clone()
+        scaled = hip.linear_into_residual(hip.pending_linear(x[:m].contiguous(), w), r, gain, 1e-5)
+        assert isinstance(scaled, ScaledRows)
+        return r, scaled.rows, hip.gated_linear(scaled, w_gu), hip.linear(scaled, w_gu)
+    full = through(16)
+    for m in (1, 4, 5, 11):
+        for got, want in zip(through(m), full):
+            assert torch.equal(got, want[:m]), m
+
+
 @pytest.mark.parametrize("q_len, kv_len, window", [(130, 130, None), (900, 1000, None), (1900, 1900, None),
                                                   (1900, 2100, 300)])
 def test_matrix_core_prefill_in_each_workgroup_shape(hip, q_len, kv_len, window):
@@ -428,7 +508,8 @@ def test_matrix_core_attention_runs_longer_than_a_block_table_window(hip, monkey
     token over 17,500 keys (four runs of about 4,380 keys), and a prompt portion under a window of 5,000."""
     n_heads, n_kv, D, ps = 2, 1, 16, 64
     dtype = torch.bfloat16
-    monkeypatch.setattr(type(hip), "decode_split", staticmethod(lambda n_seqs, n_kv_heads, kv_bound: 1))
+    # one workgroup per (sequence, kv head), whatever the length: a wave's run of keys is then longer than a window
+    monkeypatch.setattr(hip._attn_lib(D), "sia_attn_decode_max_splits", lambda kv_bound, window: 1)
     for q_lens, kv_lens, window in (([1], [17500], None), ([1], [17500], 9001), ([70], [9000], 5000)):
         ctx = Ctx(q_lens, kv_lens)
         cache = Cache(-(-kv_lens[0] // ps) + 3, n_kv, ps, D, dtype, kv_lens, seed=21)

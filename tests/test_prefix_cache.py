@@ -27,7 +27,7 @@ def test_match_shares_complete_pages_and_clear_keeps_live_requests():
     pc.insert([1, 2, 3, 4], m.table(0, 1))
     assert m.free_pages() == 4
     pages = pc.match([1, 2, 3, 4, 5])
-    assert pages == m.table(0, 1) and pc.stats()["matched_tokens"] == 4
+    assert pages == m.table(0, 1) and pc.stats()["tokens_reused"] == 4
     assert pc.match([1, 2, 3, 4]) == m.table(0, 1)[:1]          # a token must be left to run
     assert pc.match([9, 9, 9]) == []
     m.admit(2, total_tokens=6, shared_pages=pages)
@@ -51,10 +51,49 @@ def test_least_recently_used_leaf_goes_first():
         pc.insert(toks, m.table(0, rid))
         m.release(rid)
     assert pc.match([1, 2, 3, 4, 0]) == [] and len(pc.match([5, 6, 7, 8, 0])) == 2
-    assert pc.stats()["evictions"] == 2 and pc.stats()["cached_blocks"] == 2
+    assert pc.stats()["pages_dropped"] == 2 and pc.stats()["pages"] == 2 and len(pc) == 2
     assert m.free_pages() == 6
     assert pc.evict_until_available(8) and m.free_pages() == 8
     assert not pc.evict_until_available(9)
+
+
+def test_the_end_of_a_chain_that_was_used_longest_ago_goes_first_and_protected_pages_stay():
+    """Three prompts share their first page; what ends a chain and is oldest is dropped, an entry that others
+    continue never, a protected page never, and an entry whose last continuation went becomes an end itself."""
+    m = manager(16)
+    pc = PrefixCache(m, max_pages=16)
+    prompts = {1: [1, 2, 3, 4, 5, 6], 2: [1, 2, 7, 8], 3: [1, 2, 9, 9]}
+    tables = {}
+    for rid, toks in prompts.items():
+        m.admit(rid, total_tokens=len(toks))
+        m.extend(rid, len(toks))
+        tables[rid] = list(m.table(0, rid))
+        pc.insert(toks, tables[rid])
+        m.release(rid)
+    assert len(pc) == 5 and m.free_pages() == 16 - 7 + 2            # the two duplicates of the first page are free
+    pc.match([1, 2, 3, 4, 5, 6, 0])                                   # chain 1 is the most recently used now
+    shared = tables[1][0]
+    # oldest end is chain 2's second page; protect it: chain 3's goes instead
+    assert pc.evict_until_available(m.free_pages() + 1, protected={tables[2][1]})
+    assert pc.match([1, 2, 9, 9, 0]) == [shared] and pc.match([1, 2, 7, 8, 0]) == [shared, tables[2][1]]
+    # drop everything but keep the first page: its continuations go one by one, then it is an end itself
+    assert pc.evict_until_available(m.free_pages() + 3, protected={shared})
+    assert len(pc) == 1 and not pc.evict_until_available(m.free_pages() + 1, protected={shared})
+    assert pc.evict_until_available(16) and len(pc) == 0
+    m.check()
+
+
+def test_the_lazy_heap_is_started_afresh_when_it_is_mostly_stale():
+    m = manager(4)
+    pc = PrefixCache(m, max_pages=4)
+    m.admit(1, total_tokens=2)
+    m.extend(1, 2)
+    pc.insert([1, 2], m.table(0, 1))
+    for _ in range(500):
+        assert pc.match([1, 2, 3]) == m.table(0, 1)
+    assert len(pc._ends) <= 4 * len(pc) + 65
+    m.release(1)
+    assert pc.evict_until_available(4) and m.free_pages() == 4
 
 
 def test_refuses_models_it_cannot_serve():
@@ -83,7 +122,7 @@ def test_engine_with_prefix_reuse_gives_the_same_tokens(tmp_path):
     eng, cached_out = run(True)
     assert [g for g, _ in cached_out] == [g for g, _ in plain_out]
     assert [c for _, c in cached_out] == [0, 32, 16, 0]        # whole pages of 8, one token always left to run
-    assert eng.prefix_cache.stats()["hits"] == 2 and eng.prefix_cache.stats()["cached_blocks"] <= 6
+    assert eng.prefix_cache.stats()["lookups_hit"] == 2 and eng.prefix_cache.stats()["pages"] <= 6
     eng.cache.check()
     eng.reset()
     assert eng.cache.free_pages() == 24

@@ -11,66 +11,123 @@ from twins import TwinKernels
 
 
 def req(n_prompt, max_new=4):
-    return Request(prompt_tokens=list(range(1, n_prompt + 1)), params=SamplingParams(max_new_tokens=max_new))
+    return Request(list(range(1, n_prompt + 1)), SamplingParams(max_new_tokens=max_new))
+
+
+def ids(plan):
+    return [(r.id, n) for r, n in plan]
+
+
+def ran(plan):
+    """What the engine does with a plan, as far as the scheduler can see it: the requests take their tokens."""
+    for r, n in plan:
+        _, samples, _ = r.take(n)
+        if samples:
+            r.sampled(0)
 
 
 # ---- the scheduler alone ---------------------------------------------------------------------
-def test_admission_is_first_come_first_served_without_overtaking():
+def test_coming_in_is_first_come_first_served_without_overtaking():
     s = Scheduler(max_running=4, token_budget=1000, chunk_tokens=8)
     a, b, c = req(5), req(50), req(2)
     for r in (a, b, c):
-        s.add(r)
+        s.submit(r)
     fits = lambda r: r.prompt_len < 10          # b cannot get its pages
-    assert s.admit(fits) == [a]
+    assert s.let_in(fits) is a
     assert [r.state for r in (a, b, c)] == [RequestState.PREFILL, RequestState.WAITING, RequestState.WAITING]
-    assert s.admit(fits) == []                   # c does not jump over b
-    assert s.admit(lambda r: True) == [b, c]
+    assert s.let_in(fits) is None                # c does not jump over b
+    assert s.let_in() is b and s.let_in() is c and s.let_in() is None
+    assert s.live == [a, b, c] and not s.queue
 
 
 def test_token_budget_and_slots():
     s = Scheduler(max_running=2, token_budget=10, chunk_tokens=8)
     a, b, c = req(30), req(4), req(4)
     for r in (a, b, c):
-        s.add(r)
-    assert s.admit() == [a]                      # an idle engine always admits one, however long
-    assert s.admit() == []                       # 30 + 4 > 10
+        s.submit(r)
+    assert s.let_in() is a                       # an empty engine takes any one request, however long
+    assert s.let_in() is None                    # 30 + 4 > 10
     a.state = RequestState.FINISHED
-    assert s.evict_finished() == [a]
-    assert s.admit() == [b, c] and s.admit() == []   # two slots
+    assert s.retire() == [a] and s.retire() == []
+    assert s.let_in() is b and s.let_in() is c and s.let_in() is None   # two slots
+    with pytest.raises(ValueError):
+        s.submit(b)                              # only a waiting request can be queued
+
+
+def test_the_budget_counts_tokens_in_flight():
+    s = Scheduler(max_running=3, token_budget=12, chunk_tokens=8)
+    a, b, c = req(5, max_new=8), req(6), req(1)
+    s.submit(a), s.submit(b), s.submit(c)
+    plan = s.plan()
+    assert ids(plan) == [(a.id, 5), (b.id, 3)] and c.state is RequestState.WAITING   # 5 + 6 + 1 = 12 would fit, but
+    ran(plan)                                                                       # the step's room was used up
+    assert a.context_len == 6                    # its sampled token is in flight and counts
+    assert s.let_in() is None                    # 6 + 6 + 1 > 12
+    a.state = RequestState.FINISHED
+    s.retire()
+    assert s.let_in() is c
 
 
 def test_plan_gives_decoders_one_token_then_prompt_portions_in_order():
     s = Scheduler(max_running=4, token_budget=1000, chunk_tokens=8)
     d1, d2, p1, p2 = req(3), req(3), req(20), req(5)
     for r in (d1, p1, d2, p2):
-        s.add(r)
-    s.admit()
-    d1.state = d2.state = RequestState.DECODE
-    p1.num_computed = 16
-    plan = s.plan_step()
-    assert [(r.id, n) for r, n in plan] == [(d1.id, 1), (d2.id, 1), (p1.id, 4), (p2.id, 2)]
-    p1.num_computed, p2.num_computed = 20, 2
-    p1.state = RequestState.DECODE
-    assert [(r.id, n) for r, n in s.plan_step()] == [(d1.id, 1), (p1.id, 1), (d2.id, 1), (p2.id, 3)]
+        s.submit(r)
+    while s.let_in():
+        pass
+    ran([(d1, 3), (d2, 3), (p1, 16)])
+    plan = s.plan(admit=False)
+    assert ids(plan) == [(d1.id, 1), (d2.id, 1), (p1.id, 4), (p2.id, 2)]
+    ran(plan)
+    assert p1.state is RequestState.DECODE and p2.num_computed == 2
+    assert ids(s.plan(admit=False)) == [(d1.id, 1), (p1.id, 1), (d2.id, 1), (p2.id, 3)]
 
 
-def test_plan_admits_newcomers_only_into_room_for_their_first_tokens():
+def test_plan_lets_newcomers_in_only_where_there_is_room_for_their_first_tokens():
     s = Scheduler(max_running=4, token_budget=1000, chunk_tokens=8)
     a, b, c, d = req(11), req(3), req(6), req(2)
     for r in (a, b, c, d):
-        s.add(r)
-    plan = s.plan_step(admit=True)
-    assert [(r.id, n) for r, n in plan] == [(a.id, 8)]          # a fills the step: nobody else enters yet
+        s.submit(r)
+    plan = s.plan()
+    assert ids(plan) == [(a.id, 8)]                              # a fills the step: nobody else enters yet
     assert [r.state for r in (a, b, c)] == [RequestState.PREFILL, RequestState.WAITING, RequestState.WAITING]
-    a.num_computed = 8
-    plan = s.plan_step(admit=True)                               # a's rest, all of b, the start of c
-    assert [(r.id, n) for r, n in plan] == [(a.id, 3), (b.id, 3), (c.id, 2)]
-    assert d.state is RequestState.WAITING and len(s.running) == 3
-    # the admission test still decides, and nobody overtakes the head of the queue
-    a.num_computed, b.num_computed, c.num_computed = 11, 3, 6
-    a.state = b.state = c.state = RequestState.DECODE
-    assert [(r.id, n) for r, n in s.plan_step(lambda r: False)] == [(a.id, 1), (b.id, 1), (c.id, 1)]
-    assert [(r.id, n) for r, n in s.plan_step(lambda r: True)] == [(a.id, 1), (b.id, 1), (c.id, 1), (d.id, 2)]
+    ran(plan)
+    plan = s.plan()                                              # a's rest, all of b, the start of c
+    assert ids(plan) == [(a.id, 3), (b.id, 3), (c.id, 2)]
+    assert d.state is RequestState.WAITING and len(s.live) == 3
+    ran(plan)
+    ran([(c, 4)])
+    # the gate still decides, and nobody overtakes the head of the queue
+    assert ids(s.plan(lambda r: False)) == [(a.id, 1), (b.id, 1), (c.id, 1)]
+    assert ids(s.plan(admit=False)) == [(a.id, 1), (b.id, 1), (c.id, 1)]
+    assert ids(s.plan(lambda r: True)) == [(a.id, 1), (b.id, 1), (c.id, 1), (d.id, 2)]
+
+
+def test_a_request_keeps_its_own_books():
+    r = req(5, max_new=2)
+    assert r.tokens_wanted(8) == 0 and r.total_len == 7      # waiting: it brings nothing
+    r.enter(slot=3, reused_tokens=2)
+    assert (r.state, r.slot, r.num_computed, r.cached_prefix_len) == (RequestState.PREFILL, 3, 2, 2)
+    assert r.tokens_wanted(2) == 2 and r.tokens_wanted(99) == 3
+    assert r.take(2) == ([3, 4], False, None)
+    with pytest.raises(ValueError):
+        r.take(2)                                            # one token is left
+    assert r.take(1) == ([5], True, None)
+    r.sampled(row=4)
+    assert r.state is RequestState.DECODE and r.context_len == 6 and r.length_is_certain_after_next_token()
+    assert r.take(1) == ([0], True, 4)                       # its input is still on the device, in row 4
+    r.sampled(row=0)
+    assert not r.length_is_certain_after_next_token()
+    assert r.deliver(9) and r.generated == [9] and r.state is RequestState.DECODE
+    assert r.deliver(2, eos_ids=(2,)) and r.eos_hit and r.state is RequestState.FINISHED and r.slot is None
+    r.in_flight = 1
+    assert not r.deliver(11) and r.generated == [9, 2]       # sampled a step too far: dropped
+    q = req(1, max_new=1)
+    q.enter(0)
+    q.take(1), q.sampled(0)
+    assert q.deliver(2, eos_ids=()) and q.finish_reason == "length"
+    with pytest.raises(ValueError):
+        req(3).take(1)                                       # not admitted
 
 
 # ---- the engine on the CPU -----------------------------------------------------------------------
@@ -241,3 +298,65 @@ def test_running_ahead_books_the_same_tokens_and_pages(folder):
     assert ahead_way == plain_way
     assert plain_way[0] == first[:first.index(stop) + 1]          # ended on the end-of-sequence token
     assert len(plain_way[2]) == 20 and len(plain_way[4]) == 15     # ended by count
+
+
+@pytest.mark.parametrize("chunk_tokens", [1, 4])
+def test_a_step_budget_at_or_below_the_slots_feeds_prompts_token_by_token(folder, chunk_tokens):
+    want = [plain_greedy(folder, p, 5) for p in PROMPTS[:3]]
+    eng = engine(folder, max_running=4, chunk_tokens=chunk_tokens)
+    reqs = [eng.add_request(p, max_new_tokens=5) for p in PROMPTS[:3]]
+    steps = 0
+    while eng.has_work():
+        eng.step()
+        steps += 1
+        assert steps < 500
+    assert [r.generated for r in reqs] == want
+    eng.cache.check()
+
+
+def test_named_ranges_wrap_the_phases_of_a_step(folder):
+    eng = engine(folder, profile_ranges=True)
+    eng.add_request(PROMPTS[1], max_new_tokens=2)
+    eng.run()
+    names = eng.ranges.entered
+    assert names[:2] == ["engine.schedule", "engine.forward"]
+    assert all(names[i - 1] == "engine.forward" for i, n in enumerate(names) if n == "engine.sample")
+    assert {"engine.schedule", "engine.forward", "engine.sample", "engine.collect"} <= set(names)
+    off = engine(folder)
+    off.add_request(PROMPTS[1], max_new_tokens=2)
+    off.run()
+    assert off.ranges.entered == []
+
+
+def test_the_engine_goes_on_eagerly_when_its_graphs_give_up(folder, capsys):
+    """The engine's side of the fallback, with a stand-in for the graphs (the real ones need a GPU): a stand-in
+    that books a step as the real one does, then fails and takes its booking back."""
+    from simple_inference_amd.engine.graphs import GraphUnavailable
+
+    class GraphsThatFail:
+        def __init__(self, eng, after):
+            self.eng, self.after, self.calls = eng, after, 0
+
+        def can_run(self, entries):
+            return all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+
+        def run(self, entries, device_tokens=None):
+            self.calls += 1
+            if self.calls <= self.after:
+                return self.eng.runner.run(entries, device_tokens)
+            for e in entries:
+                self.eng.cache.extend(e.req, 1)
+            for e in entries:
+                self.eng.cache.retract(e.req, 1)
+            raise GraphUnavailable("made up by the test") from RuntimeError("replay refused")
+
+    want = [plain_greedy(folder, p, 6) for p in PROMPTS[:3]]
+    eng = engine(folder, max_running=4)
+    eng.graphs = GraphsThatFail(eng, after=2)
+    reqs = [eng.add_request(p, max_new_tokens=6) for p in PROMPTS[:3]]
+    eng.run()
+    assert [r.generated for r in reqs] == want
+    assert eng.graphs is None and eng.stats["graph_fallbacks"] == 1
+    assert "replay refused" in capsys.readouterr().err
+    eng.cache.check()
+    assert eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks()
