@@ -46,6 +46,7 @@ _SIGNATURES = {
     "sia_gemm_skinny_residual": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "sia_place_tokens": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "sia_scale_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr],
+    "sia_stream_read": [_c_ptr, _c_ll, _c_ptr, _c_ptr],
 }
 
 
@@ -194,6 +195,24 @@ class HipKernels:
             raise KernelError(f"{what} must be {dtype}, is {t.dtype}")
         if shape is not None and tuple(t.shape) != tuple(shape):
             raise KernelError(f"{what} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+
+    # -- measurement -----------------------------------------------------------
+    def measured_read_bandwidth(self, megabytes: int = 2048, repeats: int = 5) -> float:
+        """GB/s that a plain streaming read of a buffer far larger than the caches reaches on this card (the best
+        of ``repeats``): the ceiling a decode step's reads can be priced against beside the published one."""
+        n = int(megabytes) * (1 << 20)
+        buf = torch.empty(n, dtype=torch.uint8, device=self.device)
+        buf.zero_()
+        sink = torch.zeros(1, dtype=torch.int32, device=self.device)
+        best = 0.0
+        for _ in range(repeats + 1):   # the first run warms up
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            self._check(self.core.sia_stream_read(_ptr(buf), n, _ptr(sink), self._stream()), "stream_read")
+            end.record()
+            end.synchronize()
+            best = max(best, n / (start.elapsed_time(end) * 1e-3) / 1e9)
+        return best
 
     # -- embedding -------------------------------------------------------------
     def place_tokens(self, token_ids, dst_rows, src_tokens, src_rows):

@@ -159,8 +159,9 @@ def block(x, positions, w, i, cfg, inv_freq):
     return x
 
 
-def forward(cfg, w, tokens, start_position=0):
-    """Logits [T, V] of one whole sequence.  reference: model/llama.py:173-186 —
+def forward(cfg, w, tokens, start_position=0, rows=None):
+    """Logits [T, V] of one whole sequence (with ``rows``: at those places only, [len(rows), V]; the layers
+    still see the whole sequence).  reference: model/llama.py:173-186 —
     embed -> blocks -> norm -> head; tied head = embedding matrix (ops/embedding.py:84-92)."""
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(start_position, start_position + len(tokens))
@@ -168,6 +169,8 @@ def forward(cfg, w, tokens, start_position=0):
     x = w["model.embed_tokens.weight"][tokens]
     for i in range(cfg["num_hidden_layers"]):
         x = block(x, positions, w, i, cfg, inv_freq)
+    if rows is not None:
+        x = x[torch.as_tensor(rows, dtype=torch.long)]
     x = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", True) else w["lm_head.weight"]
     return x @ head.T

@@ -1,0 +1,216 @@
+"""The whole engine at real layer widths against the plain implementation.
+
+Two layers of each of the three shapes the presets name (the widths, head counts, head sizes, vocabulary and
+frequency scaling of the 3B, 1B and 8B models; fewer layers, so that the plain implementation on the CPU takes
+seconds), with seeded random weights, in float32 and in bfloat16.  At these widths the engine takes the paths the
+tiny models never reach together: the few-row products with fused epilogues at K of 3,072 to 14,336 in their
+16-wave shapes, the BLAS library from 17 rows on, the matrix-core attention of head sizes 128 and 64 with groups
+of 3 and 4, key splits of 1 to 8 workgroups, a vocabulary of 128,256 (reference:
+``benchmarks/bench_paged_cudagraph.py:236-264`` compares its fast path's logits at the real model the same way).
+"""
+
+import copy
+
+import pytest
+import torch
+
+import plain_llama as plain
+from helpers import TOLERANCE, random_tokens, rel_err
+from simple_inference_amd import preset
+from simple_inference_amd.engine import StepEntry
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = {"3b": "llama-3.2-3b", "1b": "llama-3.2-1b", "8b": "llama-3.1-8b"}
+LAYERS = 2
+PAGE = 16
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """name -> (folder, plain config, plain weights); written and read once for all tests of the module."""
+    made = {}
+
+    def get(name):
+        if name not in made:
+            from simple_inference_amd.config import EngineConfig
+            from simple_inference_amd.engine import build_model
+            from simple_inference_amd.weights import random_tensors, write_model_folder
+            cfg = preset(SHAPES[name])
+            cfg["num_hidden_layers"] = LAYERS
+            cfg["max_position_embeddings"] = 8192
+            model, mcfg = build_model(cfg, EngineConfig(device="cpu", dtype="float32", max_seq_len=64), kernels=None)
+            tensors = random_tensors(model.expected_tensors(), seed=7, std=0.02, gain_std=0.1, device="cuda:0")
+            folder = write_model_folder(tmp_path_factory.mktemp(f"real_{name}"), mcfg.to_dict(), tensors)
+            del tensors
+            made[name] = (folder,) + plain.read_model(folder)
+        return made[name]
+    return get
+
+
+_plain_rows = {}
+
+
+def plain_rows(models, name, tokens, rows):
+    """The plain implementation's logits of ``tokens`` at ``rows`` (kept: both dtypes ask for the same)."""
+    key = (name, tuple(tokens), tuple(rows))
+    if key not in _plain_rows:
+        _, cfg, w = models(name)
+        _plain_rows[key] = plain.forward(cfg, w, tokens, rows=list(rows))
+    return _plain_rows[key]
+
+
+def runner_for(models, name, dtype, num_pages, max_seq_len=512, max_running=4):
+    from simple_inference_amd.cache import CacheManager
+    from simple_inference_amd.config import EngineConfig
+    from simple_inference_amd.engine import StepRunner, model_from_folder
+    from simple_inference_amd.kernels import HipKernels
+    kernels = HipKernels()
+    ecfg = EngineConfig(device="cuda:0", dtype=dtype, max_seq_len=max_seq_len, block_size=PAGE,
+                        num_kv_blocks=num_pages, max_running=max_running)
+    model, mcfg = model_from_folder(models(name)[0], ecfg, kernels)
+    cache = CacheManager(model.cache_layout(), page_size=PAGE, num_pages=num_pages, max_running=max_running,
+                         dtype=ecfg.torch_dtype, device="cuda:0")
+    return StepRunner(model, cache, kernels, "cuda:0", max_seq_len), cache, kernels
+
+
+def run_schedule(runner, cache, schedule):
+    """schedule: steps of (entries, ends), an entry (request, tokens, wanted places).  {request: {position: row}}."""
+    got, fed = {}, {}
+    for entries, ends in schedule:
+        batch = []
+        for req, tokens, want in entries:
+            if req not in cache.lengths:
+                cache.admit(req)
+                fed[req] = 0
+            batch.append(StepEntry(req, tokens, want))
+        logits = runner.run(batch)
+        r = 0
+        for req, tokens, want in entries:
+            for w in want:
+                got.setdefault(req, {})[fed[req] + w] = logits[r].float().cpu()
+                r += 1
+            fed[req] += len(tokens)
+        for req in ends:
+            cache.release(req)
+        cache.check()
+    return got
+
+
+def worst_error(models, name, got, prompts):
+    worst, top1 = 0.0, []
+    for req, rows in got.items():
+        pos = sorted(rows)
+        ref = plain_rows(models, name, prompts[req], pos)
+        mine = torch.stack([rows[p] for p in pos])
+        worst = max(worst, rel_err(mine, ref))
+        top1 += (mine.argmax(-1) == ref.argmax(-1)).tolist()
+    return worst, sum(top1) / len(top1)
+
+
+def cut(tokens, sizes):
+    out, i, k = [], 0, 0
+    while i < len(tokens):
+        n = min(sizes[k % len(sizes)], len(tokens) - i)
+        out.append(tokens[i:i + n])
+        i += n
+        k += 1
+    return out
+
+
+def the_four_cuts(vocab):
+    """One schedule with all four ways of cutting: a prompt whole; most of one in a step and its last 32 tokens one
+    by one; one in portions of changing size, down to two tokens; five more mixed, up to four live, portions of
+    some beside single tokens of others, in a pool so small that pages are used again."""
+    prompts = {"whole": random_tokens(vocab, 200, seed=1), "tail": random_tokens(vocab, 160, seed=2),
+               "cuts": random_tokens(vocab, 150, seed=3)}
+    schedule = [([("whole", prompts["whole"], [0, 1, 15, 16, 17, 63, 64, 127, 128, 199])], ["whole"])]
+    t = prompts["tail"]
+    schedule.append(([("tail", t[:128], [127])], []))
+    schedule += [([("tail", [t[i]], [0])], ["tail"] if i == 159 else []) for i in range(128, 160)]
+    parts = cut(prompts["cuts"], [2, 7, 3, 16, 2, 33, 5, 64, 9])
+    schedule += [([("cuts", p, list(range(len(p))))], ["cuts"] if i == len(parts) - 1 else [])
+                 for i, p in enumerate(parts)]
+    lengths = (70, 45, 90, 33, 64)
+    mixed = {f"m{i}": random_tokens(vocab, n, seed=10 + i) for i, n in enumerate(lengths)}
+    prompts.update(mixed)
+    plans = {r: cut(toks[:-5], [13 + i, 2, 7, 31]) + [[x] for x in toks[-5:]] for i, (r, toks) in enumerate(mixed.items())}
+    waiting, live, step = list(mixed), [], 0
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries, ends = [], []
+        for r in list(live):
+            if (step + int(r[1:])) % 4 == 3 and len(live) > 1:
+                continue      # left out of this step
+            part = plans[r].pop(0)
+            entries.append((r, part, list(range(len(part)))))
+            if not plans[r]:
+                ends.append(r)
+                live.remove(r)
+        schedule.append((entries, ends))
+        step += 1
+    pool = sum(sorted(-(-n // PAGE) for n in lengths)[-4:]) + 1     # the four largest of the mixed ones
+    return prompts, schedule, max(pool, -(-200 // PAGE))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["3b", "1b", "8b"])
+def test_the_four_cuts_at_real_widths(models, name, dtype):
+    vocab = models(name)[1]["vocab_size"]
+    prompts, schedule, pool = the_four_cuts(vocab)
+    runner, cache, _ = runner_for(models, name, dtype, num_pages=pool)
+    got = run_schedule(runner, cache, schedule)
+    assert sum(len(v) for v in got.values()) == 10 + 33 + 150 + 302
+    worst, top1 = worst_error(models, name, got, prompts)
+    backend = "hip-f32" if dtype == "float32" else "hip-bf16"
+    assert worst <= TOLERANCE[backend], f"{name} {dtype}: worst relative difference {worst:.3e}"
+    assert cache.free_pages() == pool
+    if dtype == "float32":
+        assert top1 == 1.0
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16", "bfloat16-unfused"])
+def test_steps_of_1_8_16_17_and_64_single_tokens_at_3b_widths(models, mode):
+    """64 requests with prompts of 3 to 34 tokens decode together, then 17, 16, 8 and one of them: a step of up to
+    16 rows takes this package's products (with the fused epilogues, or, in the third mode, without: product,
+    rotation and cache write, norm and activation as kernels of their own), from 17 rows on the BLAS library."""
+    dtype = "float32" if mode == "float32" else "bfloat16"
+    _, cfg, _ = models("3b")
+    vocab = cfg["vocab_size"]
+    prompts = {i: random_tokens(vocab, 3 + (i * 7) % 32 + 5, seed=300 + i) for i in range(64)}
+    pool = sum(-(-len(p) // PAGE) for p in prompts.values())
+    runner, cache, kernels = runner_for(models, "3b", dtype, num_pages=pool, max_running=64)
+    if mode.endswith("unfused"):
+        kernels.fuse_norms = kernels.fuse_rope = False
+    ids = list(prompts)
+    schedule = []
+    for first in range(0, 64, 16):      # the prompts, sixteen at a time, all but their last five tokens
+        schedule.append(([(i, prompts[i][:-5], []) for i in ids[first:first + 16]], []))
+    for step, group in enumerate((ids, ids[:17], ids[:16], ids[:8], ids[:1])):
+        schedule.append(([(i, [prompts[i][len(prompts[i]) - 5 + step]], [0]) for i in group], []))
+    got = run_schedule(runner, cache, schedule)
+    assert sum(len(v) for v in got.values()) == 64 + 17 + 16 + 8 + 1
+    worst, top1 = worst_error(models, "3b", got, prompts)
+    assert worst <= TOLERANCE["hip-f32" if dtype == "float32" else "hip-bf16"], f"{mode}: {worst:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_context_past_4096_tokens_crosses_every_number_of_key_splits(models, dtype):
+    """One request grows to 4,100 tokens: portions bring it to just below 512, 1,024, 2,048 and 4,096 keys, and
+    three single tokens then cross each of these lengths, at which the decode kernel shares a sequence between 1,
+    2, 4 and 8 workgroups."""
+    _, cfg, _ = models("3b")
+    tokens = random_tokens(cfg["vocab_size"], 4100, seed=400)
+    runner, cache, _ = runner_for(models, "3b", dtype, num_pages=-(-4100 // PAGE) + 1, max_seq_len=4352, max_running=2)
+    schedule, at = [], 0
+    for edge in (512, 1024, 2048, 4096):
+        for part in cut(tokens[at:edge - 2], [2048]):
+            schedule.append(([(0, part, [len(part) - 1])], []))
+        schedule += [([(0, [tokens[i]], [0])], []) for i in range(edge - 2, edge + 2)]
+        at = edge + 2
+    schedule.append(([(0, tokens[at:], [len(tokens) - at - 1])], [0]))
+    got = run_schedule(runner, cache, schedule)
+    assert sorted(got[0])[-1] == 4099 and len(got[0]) == 4 * 4 + 4 + 1
+    worst, top1 = worst_error(models, "3b", got, {0: tokens})
+    assert worst <= TOLERANCE["hip-f32" if dtype == "float32" else "hip-bf16"], f"{dtype}: {worst:.3e}"
