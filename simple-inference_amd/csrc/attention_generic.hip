@@ -87,6 +87,9 @@ __global__ __launch_bounds__(SIA_WAVE) void attention_generic_kernel(
     }
 }
 
+// The largest head size any attention kernel of this package takes (a model is checked against it when it is built).
+SIA_EXPORT int sia_attention_max_head_dim() { return ATTN_MAX_HEAD_DIM; }
+
 SIA_EXPORT int sia_attention_generic(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                                      const int* block_table, int table_width, const int* seq_of_token,
                                      const int* positions, void* out, int n_tokens, int n_heads, int n_kv,

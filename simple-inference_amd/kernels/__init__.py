@@ -33,6 +33,7 @@ _SIGNATURES = {
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_attention_generic": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "sia_attention_max_head_dim": [],
     "sia_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_sample": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "sia_sample_workspace_bytes": [_c_int],
@@ -464,6 +465,17 @@ class HipKernels:
                               f"{ctx.max_kv_len} positions with pages of {page_size}")
 
     # -- attention ---------------------------------------------------------------
+    def check_attention_geometry(self, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
+        """Raises for head counts and sizes that no attention kernel here takes.  A mixer calls it when the model is
+        built, so that such a model is refused before it is loaded, not at its first step."""
+        limit = self.core.sia_attention_max_head_dim()
+        if not 0 < head_dim <= limit:
+            raise KernelError(f"head size {head_dim} is outside what the attention kernels take (1 to {limit})")
+        if n_kv_heads <= 0 or n_heads <= 0 or n_heads % n_kv_heads:
+            raise KernelError(f"{n_heads} query heads cannot share {n_kv_heads} key/value heads evenly")
+        if n_heads > 65535:
+            raise KernelError(f"{n_heads} query heads exceed the kernels' grids (65,535)")
+
     def paged_attention(self, qkv, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
         self._want(qkv, "qkv")
         n, width = qkv.shape

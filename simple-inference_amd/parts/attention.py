@@ -54,6 +54,9 @@ class Attention:
         self.position = _shared_position_encoding(params.get("position", {"kind": "none", "params": {}}), env)
         if self.position.rotary_dim > self.head_dim:
             raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds head_dim {self.head_dim}")
+        check = getattr(env.kernels, "check_attention_geometry", None)
+        if check is not None:     # sizes the kernels refuse are refused here, when the model is built
+            check(self.num_heads, self.num_kv_heads, self.head_dim)
         self.env = env
         self.w_qkv = None
         self.w_o = None

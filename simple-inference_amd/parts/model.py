@@ -14,9 +14,8 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from .context import BuildEnv, LayerCache, ResidualStream, StepContext
-from .embedding import OutputHead, TokenEmbedding
 from .plan import ModelPlan, PagedKVNeed, StateNeed, TensorSpec
-from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS
 
 
 @dataclass
@@ -56,10 +55,14 @@ class DecoderModel:
         self.env = env
         self.hidden_size = plan.hidden_size
         self.vocab_size = plan.vocab_size
-        self.embedding = TokenEmbedding(plan.embedding.params, env)
+        self.embedding = EMBEDDINGS.get(plan.embedding.kind)(plan.embedding.params, env)
         self.layers = [_Layer(spec, env) for spec in plan.layers]
         self.final_norm = NORMS.get(plan.final_norm.kind)(plan.final_norm.params, env)
-        self.head = OutputHead(plan.head.params, env, self.embedding)
+        self.head = HEADS.get(plan.head.kind)(plan.head.params, env)
+        if plan.head.params.get("tied"):
+            if not hasattr(self.head, "share_embedding"):
+                raise ValueError(f"the plan ties a {plan.head.kind!r} head to the embedding, but that head cannot share one")
+            self.head.share_embedding(self.embedding)
         self.order = plan.run_order()
         self._parts = [(self.embedding, plan.embedding)]
         for layer in self.layers:

@@ -1,4 +1,4 @@
-"""Registries of part kinds: mixers, feed-forwards, norms, position encodings, blocks.
+"""Registries of part kinds: mixers, feed-forwards, norms, position encodings, blocks, embeddings, heads.
 
 A part class is registered under a ``kind``; a ``PartSpec`` names that kind.  A
 test or a user package adds a part with one ``register_*`` call and without a
@@ -19,6 +19,9 @@ Interfaces (``env`` is a ``BuildEnv``; ``ctx`` a ``StepContext``):
   ``tables(device) -> (cos, sin)`` indexed by absolute position.
 * block: ``__init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm)``,
   ``forward(stream, ctx, cache) -> None``.
+* embedding: ``forward(ctx) -> Tensor[N, hidden]`` float32, the residual stream's start.
+* head: ``forward(h) -> Tensor[rows, vocab]`` float32 logits; a head that can use the embedding's
+  matrix has ``share_embedding(embedding)``, called before ``bind`` when its params say ``tied``.
 """
 
 from __future__ import annotations
@@ -59,9 +62,13 @@ FEED_FORWARDS = _Registry("feed-forward")
 NORMS = _Registry("norm")
 POSITION_ENCODINGS = _Registry("position encoding")
 BLOCKS = _Registry("block")
+EMBEDDINGS = _Registry("embedding")
+HEADS = _Registry("head")
 
 register_mixer: Callable = MIXERS.register
 register_feed_forward: Callable = FEED_FORWARDS.register
 register_norm: Callable = NORMS.register
 register_position_encoding: Callable = POSITION_ENCODINGS.register
 register_block: Callable = BLOCKS.register
+register_embedding: Callable = EMBEDDINGS.register
+register_head: Callable = HEADS.register

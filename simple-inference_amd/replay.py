@@ -33,6 +33,7 @@ class TraceReplayer:
             device=device, dtype=dtype, block_size=page, num_kv_blocks=num_pages, max_running=max_live,
             max_seq_len=min(max_pos, max(max_tokens, page)))
         self.kernels = kernels if kernels is not None else default_kernels()
+        self.architecture = (cfg.get("architectures") or ["?"])[0]
         self.model, self.model_cfg = model_from_folder(model_folder, self.engine_cfg, self.kernels)
         self.cache = CacheManager(
             self.model.cache_layout(), page_size=page, num_pages=num_pages, max_running=max_live,
@@ -42,7 +43,7 @@ class TraceReplayer:
         self._next = 1
 
     def describe(self) -> str:
-        return (f"{self.model_cfg.architecture}, dtype {self.engine_cfg.dtype}, {self.engine_cfg.num_kv_blocks} "
+        return (f"{self.architecture}, dtype {self.engine_cfg.dtype}, {self.engine_cfg.num_kv_blocks} "
                 f"pages of {self.engine_cfg.block_size} tokens, kernels {getattr(self.kernels, 'name', '?')}")
 
     def step(self, entries: Sequence[dict], end: Sequence = ()) -> Optional[torch.Tensor]:

@@ -376,3 +376,252 @@ def test_feed_forward_norm_and_position_encoding_of_other_kinds(backend):
         FEED_FORWARDS.unregister("test_top_one")
         NORMS.unregister("test_centered")
         POSITION_ENCODINGS.unregister("test_linear_angles")
+
+
+# ---- an embedding and a head of other kinds, a cache of two widths, a state that does not start at zero ----------
+class ScaledEmbedding:
+    """Rows of the table times a constant (as some architectures scale their embeddings by sqrt(hidden))."""
+
+    def __init__(self, params, env):
+        self.vocab, self.hidden, self.factor = int(params["vocab_size"]), int(params["hidden_size"]), float(params["factor"])
+        self.env = env
+
+    def weight_specs(self):
+        return {"weight": TensorSpec((self.vocab, self.hidden))}
+
+    def bind(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, ctx):
+        return self.env.kernels.embed(ctx.token_ids, self.weight) * self.factor
+
+
+class SoftCappedHead:
+    """logits = cap * tanh(h W^T / cap), with a matrix of its own or the embedding's."""
+
+    def __init__(self, params, env):
+        self.vocab, self.hidden = int(params["vocab_size"]), int(params["hidden_size"])
+        self.cap, self.tied, self.env = float(params["cap"]), bool(params.get("tied")), env
+        self.embedding = None
+
+    def share_embedding(self, embedding):
+        self.embedding = embedding
+
+    def weight_specs(self):
+        return {} if self.tied else {"weight": TensorSpec((self.vocab, self.hidden))}
+
+    def bind(self, tensors):
+        self.own = tensors.get("weight")
+
+    def forward(self, h):
+        w = self.embedding.weight if self.tied else self.own
+        return self.cap * torch.tanh(self.env.kernels.linear(h, w, out_float32=True) / self.cap)
+
+
+class RunningMaxMixer:
+    """out[t] = W . max(h[0..t]) elementwise: a state that must start far below zero, not at it."""
+
+    START = -1.0e30
+
+    def __init__(self, params, env):
+        self.hidden, self.env = int(params["hidden_size"]), env
+
+    def weight_specs(self):
+        return {"w": TensorSpec((self.hidden, self.hidden))}
+
+    def bind(self, tensors):
+        self.w = tensors["w"]
+
+    def cache_need(self):
+        return None
+
+    def state_need(self):
+        return StateNeed((self.hidden,), "float32", init=self.START)
+
+    def forward(self, h, ctx, cache):
+        out = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+        slots = ctx.state_slots.tolist()
+        t = 0
+        for s, n in enumerate(ctx.q_lens):
+            running = cache.state[slots[s]]
+            for _ in range(n):
+                torch.maximum(running, h[t].float(), out=running)
+                out[t] = running
+                t += 1
+        return self.env.kernels.linear(out.to(h.dtype), self.w)
+
+
+class NarrowValueMixer:
+    """Single-head attention without rotation whose cached values are narrower than its keys (as a mixer that
+    caches a compressed value would have them): keys of 16, values of 8, written to and read from the pages here,
+    with plain tensor operations.  The cache manager only has to give it pages of the two widths."""
+
+    KEY, VALUE = 16, 8
+
+    def __init__(self, params, env):
+        self.hidden, self.env = int(params["hidden_size"]), env
+
+    def weight_specs(self):
+        return {"q": TensorSpec((self.KEY, self.hidden)), "k": TensorSpec((self.KEY, self.hidden)),
+                "v": TensorSpec((self.VALUE, self.hidden)), "o": TensorSpec((self.hidden, self.VALUE))}
+
+    def bind(self, tensors):
+        self.w = tensors
+
+    def cache_need(self):
+        from simple_inference_amd.parts import PagedKVNeed
+        return PagedKVNeed(1, self.KEY, None, value_head_dim=self.VALUE)
+
+    def state_need(self):
+        return None
+
+    def forward(self, h, ctx, cache):
+        lin = self.env.kernels.linear
+        q, k, v = lin(h, self.w["q"]), lin(h, self.w["k"]), lin(h, self.w["v"])
+        assert cache.k_pages.shape[1:] == (1, cache.page_size, self.KEY)
+        assert cache.v_pages.shape[1:] == (1, self.VALUE, cache.page_size)
+        out = torch.empty((h.shape[0], self.VALUE), dtype=torch.float32, device=h.device)
+        positions, seqs = ctx.positions.tolist(), ctx.seq_of_token.tolist()
+        for t, (p, s) in enumerate(zip(positions, seqs)):      # write first: a token sees itself
+            page = int(cache.block_table[s, p // cache.page_size])
+            cache.k_pages[page, 0, p % cache.page_size] = k[t]
+            cache.v_pages[page, 0, :, p % cache.page_size] = v[t]
+        for t, (p, s) in enumerate(zip(positions, seqs)):
+            pages = cache.block_table[s, :p // cache.page_size + 1].long()
+            keys = cache.k_pages[pages, 0].reshape(-1, self.KEY)[:p + 1].float()
+            vals = cache.v_pages[pages, 0].permute(0, 2, 1).reshape(-1, self.VALUE)[:p + 1].float()
+            probs = torch.softmax(keys @ q[t].float() / 4.0, dim=0)
+            out[t] = probs @ vals
+        return lin(out.to(h.dtype), self.w["o"])
+
+
+def odd_ends_plan(cfg):
+    from simple_inference_amd.parts import PartSpec as P
+    norm = lambda name: P("rmsnorm", {"size": H, "eps": 1e-5}, {"weight": name})
+    ffn = lambda p: P("swiglu", {"hidden_size": H, "intermediate_size": 48},
+                      {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"})
+    layers = [
+        LayerSpec(mixer=P("test_running_max", {"hidden_size": H}, {"w": "l0.w"}), feed_forward=ffn("l0.ffn"),
+                  mixer_norm=norm("l0.n1"), feed_forward_norm=norm("l0.n2")),
+        LayerSpec(mixer=P("test_narrow_value", {"hidden_size": H}, {k: f"l1.{k}" for k in "qkvo"}),
+                  feed_forward=ffn("l1.ffn"), mixer_norm=norm("l1.n1"), feed_forward_norm=norm("l1.n2")),
+    ]
+    tied = bool(cfg.get("tied"))
+    return ModelPlan(
+        hidden_size=H, vocab_size=V,
+        embedding=P("test_scaled_embedding", {"vocab_size": V, "hidden_size": H, "factor": 3.0}, {"weight": "embed"}),
+        layers=layers, final_norm=norm("final"),
+        head=P("test_soft_cap", {"vocab_size": V, "hidden_size": H, "cap": 2.0, "tied": tied},
+               {} if tied else {"weight": "head"}))
+
+
+def odd_ends_reference(w, tokens, tied):
+    import plain_llama as plain
+    w = {k: v.double() for k, v in w.items()}
+    T = len(tokens)
+    x = w["embed"][tokens] * 3.0
+    h = plain.rms_norm(x, w["l0.n1"], 1e-5)
+    x = x + torch.cummax(h, dim=0).values @ w["l0.w"].T
+    x = x + plain.swiglu_mlp(plain.rms_norm(x, w["l0.n2"], 1e-5), w["l0.ffn.gate"], w["l0.ffn.up"], w["l0.ffn.down"])
+    h = plain.rms_norm(x, w["l1.n1"], 1e-5)
+    q, k, v = h @ w["l1.q"].T, h @ w["l1.k"].T, h @ w["l1.v"].T
+    scores = (q @ k.T / 4.0).masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), float("-inf"))
+    x = x + (torch.softmax(scores, -1) @ v) @ w["l1.o"].T
+    x = x + plain.swiglu_mlp(plain.rms_norm(x, w["l1.n2"], 1e-5), w["l1.ffn.gate"], w["l1.ffn.up"], w["l1.ffn.down"])
+    logits = plain.rms_norm(x, w["final"], 1e-5) @ (w["embed"] if tied else w["head"]).T
+    return 2.0 * torch.tanh(logits / 2.0)
+
+
+@pytest.fixture()
+def odd_ends_registered():
+    from simple_inference_amd.parts import EMBEDDINGS, HEADS, register_embedding, register_head
+    register_embedding("test_scaled_embedding", ScaledEmbedding, replace=True)
+    register_head("test_soft_cap", SoftCappedHead, replace=True)
+    register_mixer("test_running_max", RunningMaxMixer, replace=True)
+    register_mixer("test_narrow_value", NarrowValueMixer, replace=True)
+    register_architecture("ToyOddEnds", lambda d: d, odd_ends_plan, replace=True)
+    yield
+    unregister_architecture("ToyOddEnds")
+    EMBEDDINGS.unregister("test_scaled_embedding")
+    HEADS.unregister("test_soft_cap")
+    MIXERS.unregister("test_running_max")
+    MIXERS.unregister("test_narrow_value")
+
+
+@pytest.mark.parametrize("backend", [pytest.param("twins"), pytest.param("hip-f32", marks=pytest.mark.gpu)])
+@pytest.mark.parametrize("tied", [False, True])
+def test_embedding_head_cache_widths_and_initial_state_from_outside(odd_ends_registered, backend, tied):
+    """An embedding that scales, a head that caps its logits (with a matrix of its own, or tied), a mixer whose
+    cached values are narrower than its keys and a state that starts at -1e30: all registered here, none known to
+    the package, stepped in portions beside each other with slots and pages handed out again."""
+    runner, cache, weights = make(backend, {"architectures": ["ToyOddEnds"], "tied": tied})
+    group = cache.groups[0]
+    assert group.need.head_dim == 16 and group.need.value_dim == 8
+    assert group.k.shape[-1] == 16 and group.v.shape[-2] == 8
+    g = torch.Generator().manual_seed(2)
+    seqs = {r: torch.randint(0, V, (n,), generator=g).tolist() for r, n in ((1, 14), (2, 21), (3, 6), (4, 11))}
+    want = {r: odd_ends_reference(weights, t, tied) for r, t in seqs.items()}
+    cuts = {1: [5, 1, 8], 2: [2, 7, 1, 11], 3: [6], 4: [1, 10]}
+    got, fed, live, waiting = {r: [] for r in seqs}, {r: 0 for r in seqs}, [], list(seqs)
+    while waiting or live:
+        while waiting and len(live) < 3:        # three slots for four requests: one is used a second time
+            live.append(waiting.pop(0))
+            cache.admit(live[-1])
+        entries = []
+        for r in live:
+            n = cuts[r].pop(0)
+            entries.append(StepEntry(r, seqs[r][fed[r]:fed[r] + n], list(range(n))))
+            fed[r] += n
+        out = runner.run(entries)
+        i = 0
+        for e in entries:
+            got[e.req].append(out[i:i + len(e.tokens)])
+            i += len(e.tokens)
+        for r in [r for r in live if not cuts[r]]:
+            cache.release(r)
+            live.remove(r)
+    for r in seqs:
+        assert rel_err(torch.cat(got[r]), want[r]) <= 3e-5, r
+    cache.check()
+    assert cache.free_pages() == 32 and cache.slots.free_slots == 3
+
+
+def test_trace_replay_runs_an_architecture_whose_configuration_is_a_plain_dictionary(toy_registered, tmp_path):
+    """The replay program's driver takes the architecture from config.json alone: a registered toy whose
+    parse_config returns the dictionary itself is replayed like any other model."""
+    from simple_inference_amd.replay import TraceReplayer
+    from simple_inference_amd.weights import write_model_folder
+    from twins import TwinKernels
+    cfg = {"architectures": ["ToyForTests"], "window": None, "max_position_embeddings": 256}
+    model, _ = build_model(cfg, EngineConfig(device="cpu", dtype="float32", max_seq_len=64), kernels=None)
+    weights = random_tensors(model.expected_tensors(), seed=3, std=0.15, gain_std=0.1)
+    folder = write_model_folder(tmp_path, cfg, weights)
+    rp = TraceReplayer(folder, "float32", 64, block_size=16, device="cpu", kernels=TwinKernels())
+    assert rp.describe().startswith("ToyForTests")
+    tokens = torch.randint(0, V, (23,), generator=torch.Generator().manual_seed(0)).tolist()
+    want = toy_reference(weights, tokens, [0, 1, 2, 1], None)
+    got = [rp.step([{"id": "a", "tokens": tokens[a:b], "want": list(range(b - a))}], ["a"] if b == 23 else [])
+           for a, b in ((0, 9), (9, 11), (11, 12), (12, 23))]
+    assert rel_err(torch.cat(got), want) <= 2e-5
+    assert not rp.ids and rp.cache.free_pages() == 4
+
+
+def test_a_head_size_no_kernel_takes_is_refused_when_the_model_is_built():
+    """Not at the first launch: the mixer asks the kernels when it is built."""
+    class Kernels:
+        def check_attention_geometry(self, n_heads, n_kv_heads, head_dim):
+            if head_dim > 256:
+                raise ValueError(f"head size {head_dim} is outside what the attention kernels take")
+    from helpers import TINY_A
+    cfg = dict(TINY_A, head_dim=320)
+    with pytest.raises(ValueError, match="head size 320"):
+        build_model(cfg, EngineConfig(device="cpu", dtype="float32", max_seq_len=64), kernels=Kernels())
+    build_model(dict(TINY_A, head_dim=256), EngineConfig(device="cpu", dtype="float32", max_seq_len=64), kernels=Kernels())
+
+
+@pytest.mark.gpu
+def test_the_compiled_kernels_refuse_a_head_size_beyond_their_limit_at_build_time():
+    from helpers import TINY_A
+    from simple_inference_amd.kernels import HipKernels, KernelError
+    with pytest.raises(KernelError, match="head size 272"):
+        build_model(dict(TINY_A, head_dim=272), EngineConfig(device="cuda:0", dtype="bfloat16", max_seq_len=64), HipKernels())

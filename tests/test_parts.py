@@ -168,12 +168,16 @@ def test_embedding_and_head_parts(backend):
         token_ids = torch.tensor([330, 0, 17, 17], dtype=torch.int32, device=env.device)
     out = emb.forward(Ctx())
     assert out.dtype == torch.float32 and torch.equal(out.cpu(), as_ref(env, table)[[330, 0, 17, 17]].float())
-    tied = OutputHead({"vocab_size": 331, "hidden_size": 40, "tied": True}, env, emb)
+    tied = OutputHead({"vocab_size": 331, "hidden_size": 40, "tied": True}, env)
+    with pytest.raises(ValueError):
+        tied.bind({})                       # tied, and given no embedding to share
+    tied.share_embedding(emb)
+    tied.bind({})
     assert tied.weight_specs() == {} and tied.weight.data_ptr() == emb.weight.data_ptr()
     h = rnd(3, 40, seed=2)
     logits = tied.forward(on(env, h))
     assert logits.dtype == torch.float32 and rel_err(logits, as_ref(env, h) @ as_ref(env, table).T) <= tol(backend)
     own = rnd(331, 40, seed=3)
-    untied = OutputHead({"vocab_size": 331, "hidden_size": 40, "tied": False}, env, emb)
+    untied = OutputHead({"vocab_size": 331, "hidden_size": 40, "tied": False}, env)
     untied.bind({"weight": on(env, own)})
     assert rel_err(untied.forward(on(env, h)), as_ref(env, h) @ as_ref(env, own).T) <= tol(backend)
