@@ -143,18 +143,55 @@ __device__ __forceinline__ void load_stage(Stage& st, const bf16_t* __restrict__
     for (int db = 0; db < DBLOCKS; ++db) st.v[db] = load8(vbase + (size_t)(db * 16 + r) * ps);
 }
 
-// Masks the scores of a tile, updates the running softmax statistics of each q column, rescales the
-// accumulators and returns the tile's probabilities as the P^T operand.
+// What a wave keeps of the softmax of its q columns, per group n of 16 columns.  A column (one query) lives in the
+// four lanes r, r + 16, r + 32, r + 48, each of which sees 8 of a tile's 32 keys.
+//   m:   the column's *reference*, in units of log2: exponentials are taken as 2^(s * scale_log2 - m).  It follows
+//        the running maximum lazily: it moves up to the maximum only when the maximum has grown more than
+//        SOFTMAX_SLACK beyond it.  Exponentials are then at most 2^SOFTMAX_SLACK instead of 1, which float sums and
+//        bfloat16 probabilities hold just as well, and (m, l, acc) stay a consistent triple, so acc / l is the
+//        same value.  The same in all four lanes of a column.
+//   mu:  m, or 0 while the column has seen no key (m = -inf).
+//   l:   this lane's part of the sum of exponentials (its 8 keys of every tile); the four lanes' parts are added
+//        once, at the end (finish_sums).
+// The point of the lazy reference: a tile on which no column's reference moves (nearly all of them) costs no
+// exchange between lanes and no rescaling of the accumulators (4 * DBLOCKS registers a column group), only a
+// maximum, a multiply-add and an exponential per score.  Whether a column's reference moves depends on that
+// column's scores alone, never on its neighbours in the wave.
+constexpr float SOFTMAX_SLACK = 8.f;
+
+template <int NQ>
+struct Softmax {
+    float m[NQ], mu[NQ], l[NQ];
+    __device__ __forceinline__ void start() {
+#pragma unroll
+        for (int n = 0; n < NQ; ++n) {
+            m[n] = -INFINITY;
+            mu[n] = 0.f;
+            l[n] = 0.f;
+        }
+    }
+    // after the last tile: l becomes the column's whole sum, in every lane
+    __device__ __forceinline__ void finish_sums() {
+#pragma unroll
+        for (int n = 0; n < NQ; ++n) l[n] = column_sum(l[n]);
+    }
+};
+
+// max without the quieting of signalling NaNs that fmaxf owes the standard (scores are never NaN)
+__device__ __forceinline__ float max2(float a, float b) { return __builtin_fmaxf(a, b); }
+
+// Masks the scores of a tile, updates the softmax state of each q column, rescales the accumulators where a
+// reference moved, and returns the tile's probabilities as the P^T operand.
 //   lo[n], hi[n]: visible keys of this lane's column in group n (hi < lo: none).
-//   scale_log2 = scale * log2(e) > 0: exponentials are taken as 2^(s * scale_log2 - m), and the running
-//   maximum m is kept in those units, so a score costs one fused multiply-add and one exp2.
-// A tile that every column of the wave sees whole skips the masking, and the accumulators are rescaled
-// only when some column's maximum moved (both tests are wave-uniform).
+//   scale_log2 = scale * log2(e) > 0.
+// A tile that every column of the wave sees whole skips the masking (the test is wave-uniform).
 template <int NQ>
 __device__ __forceinline__ void softmax_update(floatx4 (&s)[NQ][2], int kb, const int (&lo)[NQ], const int (&hi)[NQ],
-                                               float scale_log2, float (&m)[NQ], float (&l)[NQ],
-                                               floatx4 (&acc)[NQ][DBLOCKS], bf16x8 (&p)[NQ]) {
+                                               float scale_log2, Softmax<NQ>& sm, floatx4 (&acc)[NQ][DBLOCKS],
+                                               bf16x8 (&p)[NQ]) {
     const int g = (threadIdx.x & 63) >> 4;
+    float top[NQ];
+    bool grew = false;
 #pragma unroll
     for (int n = 0; n < NQ; ++n) {
         if (!__all(kb >= lo[n] && kb + TILE - 1 <= hi[n])) {
@@ -166,28 +203,35 @@ __device__ __forceinline__ void softmax_update(floatx4 (&s)[NQ][2], int kb, cons
                     if (key < lo[n] || key > hi[n]) s[n][h][i] = -INFINITY;
                 }
         }
-        float mx = fmaxf(fmaxf(fmaxf(s[n][0][0], s[n][0][1]), fmaxf(s[n][0][2], s[n][0][3])),
-                         fmaxf(fmaxf(s[n][1][0], s[n][1][1]), fmaxf(s[n][1][2], s[n][1][3])));
-        mx = column_max(mx);
-        const float m_new = fmaxf(m[n], mx * scale_log2);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
-        const float alpha = fast_exp2(m[n] - m_use);
+        top[n] = max2(max2(max2(s[n][0][0], s[n][0][1]), max2(s[n][0][2], s[n][0][3])),
+                      max2(max2(s[n][1][0], s[n][1][1]), max2(s[n][1][2], s[n][1][3]))) * scale_log2;
+        grew |= top[n] > sm.m[n] + SOFTMAX_SLACK;   // also a column's first visible key (m = -inf)
+    }
+    if (__builtin_expect(__any(grew), 0)) {
+#pragma unroll
+        for (int n = 0; n < NQ; ++n) {
+            const float mx = column_max(top[n]);
+            const bool moved = mx > sm.m[n] + SOFTMAX_SLACK;
+            const float alpha = moved ? fast_exp2(sm.m[n] - mx) : 1.f;   // from -inf: 0 (there is nothing yet)
+            sm.m[n] = moved ? mx : sm.m[n];
+            sm.mu[n] = sm.m[n] == -INFINITY ? 0.f : sm.m[n];
+            sm.l[n] *= alpha;
+#pragma unroll
+            for (int db = 0; db < DBLOCKS; ++db) acc[n][db] *= alpha;
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
         float sum = 0.f;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float e = fast_exp2(fmaf(s[n][h][i], scale_log2, -m_use));
+                const float e = fast_exp2(fmaf(s[n][h][i], scale_log2, -sm.mu[n]));
                 s[n][h][i] = e;
                 sum += e;
             }
-        sum = column_sum(sum);
-        l[n] = l[n] * alpha + sum;
-        m[n] = m_new;
-        if (__any(alpha != 1.f)) {
-#pragma unroll
-            for (int db = 0; db < DBLOCKS; ++db) acc[n][db] *= alpha;
-        }
+        sm.l[n] += sum;
         uint4 u;
         u.x = pack2(s[n][0][0], s[n][0][1]);
         u.y = pack2(s[n][0][2], s[n][0][3]);
@@ -201,7 +245,7 @@ __device__ __forceinline__ void softmax_update(floatx4 (&s)[NQ][2], int kb, cons
 template <int NQ>
 __device__ __forceinline__ void compute_stage(const Stage& st, const bf16x8 (&q)[NQ][KSTEPS], int kb,
                                               const int (&lo)[NQ], const int (&hi)[NQ], float scale,
-                                              float (&m)[NQ], float (&l)[NQ], floatx4 (&acc)[NQ][DBLOCKS]) {
+                                              Softmax<NQ>& sm, floatx4 (&acc)[NQ][DBLOCKS]) {
     floatx4 s[NQ][2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -214,7 +258,7 @@ __device__ __forceinline__ void compute_stage(const Stage& st, const bf16x8 (&q)
                 s[n][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.k[h][ks], q[n][ks], s[n][h], 0, 0, 0);
     }
     bf16x8 p[NQ];
-    softmax_update<NQ>(s, kb, lo, hi, scale, m, l, acc, p);
+    softmax_update<NQ>(s, kb, lo, hi, scale, sm, acc, p);
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db)
 #pragma unroll
@@ -229,17 +273,16 @@ __device__ __forceinline__ void attend_tiles(const PageWindow& pages, int w_firs
                                              const bf16x8 (&q)[NQ][KSTEPS], const bf16_t* __restrict__ kp,
                                              const bf16_t* __restrict__ vp, int ps_log2, int n_kv, int hk,
                                              int range_lo, int range_hi, const int (&lo)[NQ], const int (&hi)[NQ],
-                                             float scale, float (&m)[NQ], float (&l)[NQ],
-                                             floatx4 (&acc)[NQ][DBLOCKS]) {
+                                             float scale, Softmax<NQ>& sm, floatx4 (&acc)[NQ][DBLOCKS]) {
     Stage a, b;
     load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, w_first, range_lo, range_hi);
     for (int kb = w_first; kb <= w_last; kb += 2 * TILE) {
         const int kb1 = min(kb + TILE, w_last);  // past the end: the last tile again, never computed
         load_stage(b, kp, vp, pages, ps_log2, n_kv, hk, kb1, range_lo, range_hi);
-        compute_stage<NQ>(a, q, kb, lo, hi, scale, m, l, acc);
+        compute_stage<NQ>(a, q, kb, lo, hi, scale, sm, acc);
         const int kb2 = min(kb + 2 * TILE, w_last);
         load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, kb2, range_lo, range_hi);
-        if (kb + TILE <= w_last) compute_stage<NQ>(b, q, kb + TILE, lo, hi, scale, m, l, acc);
+        if (kb + TILE <= w_last) compute_stage<NQ>(b, q, kb + TILE, lo, hi, scale, sm, acc);
     }
 }
 
@@ -251,7 +294,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], cons
                                              const bf16_t* __restrict__ vp, const int* __restrict__ table,
                                              int table_width, int ps_log2, int n_kv, int hk, int range_lo,
                                              int range_hi, const int (&lo)[NQ], const int (&hi)[NQ], float scale,
-                                             float (&m)[NQ], float (&l)[NQ], floatx4 (&acc)[NQ][DBLOCKS]) {
+                                             Softmax<NQ>& sm, floatx4 (&acc)[NQ][DBLOCKS]) {
     const int lane = threadIdx.x & 63;
     const int kb_first = (range_lo / TILE) * TILE, kb_last = (range_hi / TILE) * TILE;
     for (int w_first = kb_first; w_first <= kb_last;) {
@@ -260,7 +303,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], cons
         PageWindow pages;
         pages_load(pages, table, table_width, first_page, lane);
         attend_tiles<NQ>(pages, w_first, min(kb_last, w_end - TILE), q, kp, vp, ps_log2, n_kv, hk, range_lo, range_hi,
-                         lo, hi, scale, m, l, acc);
+                         lo, hi, scale, sm, acc);
         w_first = w_end;
     }
 }
@@ -316,7 +359,8 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const int my_first = t_first + (int)(((long long)wi * n_tiles) / n_waves);
     const int my_end = t_first + (int)(((long long)(wi + 1) * n_tiles) / n_waves);
 
-    float m[1] = {-INFINITY}, l[1] = {0.f};
+    Softmax<1> sm;
+    sm.start();
     floatx4 acc[1][DBLOCKS];
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) acc[0][db] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -324,15 +368,16 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     if (my_first < my_end) {  // wave-uniform
         const int w_lo = max(lo_all, my_first * TILE), w_hi = min(pos, my_end * TILE - 1);
         const int lo[1] = {r < group ? w_lo : 1}, hi[1] = {r < group ? w_hi : 0};
-        attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, m, l, acc);
+        attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, sm, acc);
     }
+    sm.finish_sums();
 
     constexpr int ROW = HD + 2;
     if (r < group) {
         float* mine = lds + (size_t)(wave * group + r) * ROW;
         if (g == 0) {
-            mine[HD] = m[0];
-            mine[HD + 1] = l[0];
+            mine[HD] = sm.m[0];
+            mine[HD + 1] = sm.l[0];
         }
 #pragma unroll
         for (int db = 0; db < DBLOCKS; ++db)
@@ -449,34 +494,51 @@ struct TileRegs {
     u32x4 v[PER_THREAD];
 };
 
-// Issues the global loads of the tile at kb.  Key chunk c is (key c / (HD/8), dims 8 (c % (HD/8)) ..);
-// value chunks are ordered (page segment, dim, group of 8 positions), so that consecutive threads read
-// consecutive 16 bytes of a page.  Keys outside [lo, hi] are clamped into it (see load_stage).
+// Where a thread's pieces of a tile lie, as far as that does not depend on the tile: worked out once per workgroup.
+// Key piece c is (key c / (HD/8) of the tile, dims 8 (c % (HD/8)) ..); value pieces are ordered (page segment, dim,
+// group of 8 positions), so that consecutive threads read consecutive 16 bytes of a page.  With that order a
+// thread's key piece and its value piece lie in the same page segment of the tile, whatever the page size, so one
+// look-up of the page serves both.
 template <int TEAM>
-__device__ __forceinline__ void tile_fetch(TileRegs<TEAM>& t, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
-                                           const PageWindow& pages, int ps_log2, int n_kv, int hk, int kb, int lo,
-                                           int hi) {
-    const int ps = 1 << ps_log2;
-    const int t_lo = max(kb, lo), t_hi = min(kb + TILE - 1, hi);
-    const int seg_keys = min(ps, TILE);            // positions of one page inside a tile
-    const int seg_chunks = HD * (seg_keys / 8);    // 16-byte pieces of one page's values inside a tile
+struct FetchPlan {
+    static constexpr int PER_THREAD = (K_CHUNKS + TEAM - 1) / TEAM;
+    int k_key[PER_THREAD], k_off[PER_THREAD];  // key within the tile; element offset of the piece within its page
+    int v_key[PER_THREAD], v_off[PER_THREAD];  // first of its 8 positions within the tile; offset within the page
+    __device__ __forceinline__ void make(int ps_log2, int hk) {
+        const int ps = 1 << ps_log2;
+        const int seg_keys = min(ps, TILE);            // positions of one page inside a tile
+        const int seg_chunks = HD * (seg_keys / 8);    // 16-byte pieces of one page's values inside a tile
 #pragma unroll
-    for (int i = 0; i < TileRegs<TEAM>::PER_THREAD; ++i) {
-        const int c = threadIdx.x + i * TEAM;
-        if (K_CHUNKS % TEAM != 0 && c >= K_CHUNKS) break;
-        {
-            const int key = min(max(kb + c / (HD / 8), t_lo), t_hi);
-            const int page = pages_get(pages, key >> ps_log2);
-            t.k[i] = *reinterpret_cast<const u32x4*>(kp + (((size_t)page * n_kv + hk) * ps + (key & (ps - 1))) * HD +
-                                                     (c % (HD / 8)) * 8);
-        }
-        {
+        for (int i = 0; i < PER_THREAD; ++i) {
+            const int c = min((int)threadIdx.x + i * TEAM, K_CHUNKS - 1);
+            k_key[i] = c / (HD / 8);
+            k_off[i] = hk * ps * HD + (c % (HD / 8)) * 8;
             const int seg = c / seg_chunks, rest = c % seg_chunks;
             const int d = rest / (seg_keys / 8), j = rest % (seg_keys / 8);
-            const int key0 = min(max(kb + seg * seg_keys + j * 8, t_lo & ~7), t_hi & ~7);
-            const int page = pages_get(pages, key0 >> ps_log2);
-            t.v[i] = *reinterpret_cast<const u32x4*>(vp + (((size_t)page * n_kv + hk) * HD + d) * ps + (key0 & (ps - 1)));
+            v_key[i] = seg * seg_keys + j * 8;
+            v_off[i] = (hk * HD + d) * ps;
         }
+    }
+};
+
+// Issues the global loads of the tile at kb.  Keys outside [lo, hi] are clamped into it (see load_stage); a key
+// piece and its value piece then still lie in one page: both are clamped into the same range, whose ends lie in
+// pages of their own only as a whole.  page_stride: elements of one page (keys and values alike).
+template <int TEAM>
+__device__ __forceinline__ void tile_fetch(TileRegs<TEAM>& t, const FetchPlan<TEAM>& plan, const bf16_t* __restrict__ kp,
+                                           const bf16_t* __restrict__ vp, const PageWindow& pages, int ps_log2,
+                                           unsigned page_stride, int kb, int lo, int hi) {
+    const int ps_mask = (1 << ps_log2) - 1;
+    const int t_lo = max(kb, lo), t_hi = min(kb + TILE - 1, hi);
+    const int v_lo = t_lo & ~7, v_hi = t_hi & ~7;
+#pragma unroll
+    for (int i = 0; i < TileRegs<TEAM>::PER_THREAD; ++i) {
+        if (K_CHUNKS % TEAM != 0 && (int)threadIdx.x + i * TEAM >= K_CHUNKS) break;
+        const int key = min(max(kb + plan.k_key[i], t_lo), t_hi);
+        const int key0 = min(max(kb + plan.v_key[i], v_lo), v_hi);
+        const size_t page_at = (size_t)(unsigned)pages_get(pages, key >> ps_log2) * page_stride;
+        t.k[i] = *reinterpret_cast<const u32x4*>(kp + page_at + (unsigned)(plan.k_off[i] + (key & ps_mask) * HD));
+        t.v[i] = *reinterpret_cast<const u32x4*>(vp + page_at + (unsigned)(plan.v_off[i] + (key0 & ps_mask)));
     }
 }
 
@@ -506,7 +568,7 @@ __device__ __forceinline__ void tile_store(const TileRegs<TEAM>& t, bf16_t* __re
 template <int NQ>
 __device__ __forceinline__ void compute_from_lds(const bf16_t* __restrict__ k_lds, const bf16_t* __restrict__ v_lds,
                                                  const bf16x8 (&q)[NQ][KSTEPS], int kb, const int (&lo)[NQ],
-                                                 const int (&hi)[NQ], float scale, float (&m)[NQ], float (&l)[NQ],
+                                                 const int (&hi)[NQ], float scale, Softmax<NQ>& sm,
                                                  floatx4 (&acc)[NQ][DBLOCKS]) {
     const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     floatx4 s[NQ][2];
@@ -527,7 +589,7 @@ __device__ __forceinline__ void compute_from_lds(const bf16_t* __restrict__ k_ld
         }
     }
     bf16x8 p[NQ];
-    softmax_update<NQ>(s, kb, lo, hi, scale, m, l, acc, p);
+    softmax_update<NQ>(s, kb, lo, hi, scale, sm, acc, p);
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) {
         const bf16x8 a = load8(v_lds + (db * 16 + r) * V_STRIDE + g * 8);
@@ -581,7 +643,8 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
 
     bf16x8 qf[PF_NQ][KSTEPS];
     int lo[PF_NQ], hi[PF_NQ];
-    float m[PF_NQ], l[PF_NQ];
+    Softmax<PF_NQ> sm;
+    sm.start();
     floatx4 acc[PF_NQ][DBLOCKS];
 #pragma unroll
     for (int n = 0; n < PF_NQ; ++n) {
@@ -591,8 +654,6 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
         load_q(qf[n], live ? q + (size_t)(q_begin + row) * q_row_stride + head * HD : nullptr, g);
         hi[n] = live ? qpos : 0;
         lo[n] = live ? (window > 0 ? max(0, qpos - window + 1) : 0) : 1;
-        m[n] = -INFINITY;
-        l[n] = 0.f;
 #pragma unroll
         for (int db = 0; db < DBLOCKS; ++db) acc[n][db] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
@@ -611,8 +672,13 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
         const int wave_lo = window > 0 ? max(0, first_pos + row0 - window + 1) : 0;
         const int kb_first = (blk_lo / TILE) * TILE, kb_last = (blk_hi / TILE) * TILE;
         constexpr int STEP_KEYS = KTILES * TILE;
-        // Two register sets: while the tiles of step t are computed from LDS, those of step t+1 wait in one set
-        // (their loads were issued a step ago) and the loads of step t+2 are issued into the other.  The
+        constexpr int AHEAD = PF_NQ == 1 ? 4 : 2;
+        static_assert(AHEAD % 2 == 0, "the LDS stage of a step is its parity within a group of AHEAD");
+        FetchPlan<TEAM> plan;
+        plan.make(ps_log2, hk);
+        const unsigned page_stride = (unsigned)n_kv * HD << ps_log2;
+        // AHEAD (two or four) register sets: while the tiles of step t are computed from LDS, those of the steps
+        // after it wait in the others (or are still on their way) and the loads of step t+AHEAD are issued.  The
         // block-table window (64 entries from the page of the first tile it serves) is loaded outside the
         // pipelined loop.
         for (int w_first = kb_first, w_end; w_first <= kb_last; w_first = w_end) {
@@ -621,36 +687,42 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
             const int w_last = min(kb_last, w_end - TILE);
             PageWindow pages;
             pages_load(pages, table, table_width, first_page, lane);
-            TileRegs<TEAM> regs_a[KTILES], regs_b[KTILES];
-// One step: issue the loads of the tiles two steps ahead into FREE, compute this wave's tile of the step at KB
-// from LDS stage STAGE, write the tiles that wait in NEXT into the other stage.  (Macros, not lambdas: register
-// sets that a closure captures by reference end up in scratch memory.)
+            TileRegs<TEAM> regs[AHEAD][KTILES];
+// One step: issue the loads of the tiles AHEAD steps ahead into FREE (whose tiles are in LDS by now), compute this
+// wave's tile of the step at KB from LDS stage STAGE, write the tiles that wait in NEXT (loaded AHEAD - 1 steps
+// ago) into the other stage.  With AHEAD = 4 a load has three steps' time to arrive before anybody waits for it:
+// with the one or two workgroups a compute unit holds when a prompt is short, nothing else would hide its latency
+// (the shapes of 32 tokens a wave have no registers to spare for it and hide it by their number).  (Macros, not
+// lambdas: register sets that a closure captures by reference end up in scratch memory.)
 #define PF_FETCH(SET, KB)                                                                                       \
     _Pragma("unroll") for (int p = 0; p < KTILES; ++p)                                                          \
-        tile_fetch(SET[p], kp, vp, pages, ps_log2, n_kv, hk, min((KB) + p * TILE, w_last), blk_lo, blk_hi)
+        tile_fetch(SET[p], plan, kp, vp, pages, ps_log2, page_stride, min((KB) + p * TILE, w_last), blk_lo, blk_hi)
 #define PF_STORE(SET, KB, STAGE)                                                                                \
     _Pragma("unroll") for (int p = 0; p < KTILES; ++p)                                                          \
         if ((KB) + p * TILE <= w_last) tile_store(SET[p], PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), ps_log2)
 #define PF_STEP(FREE, NEXT, KB, STAGE)                                                                          \
     do {                                                                                                        \
-        PF_FETCH(FREE, (KB) + 2 * STEP_KEYS);                                                                   \
+        PF_FETCH(FREE, (KB) + AHEAD * STEP_KEYS);                                                               \
         _Pragma("unroll") for (int p = 0; p < KTILES; ++p) {                                                    \
             if (p % KSPLIT != part) continue; /* each set of waves its tiles of the step */                     \
             const int my_kb = (KB) + p * TILE;                                                                  \
             if (wave_live && my_kb <= w_last && my_kb <= wave_hi && my_kb + TILE - 1 >= wave_lo)                \
-                compute_from_lds<PF_NQ>(PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), qf, my_kb, lo, hi, scale, m, l, \
+                compute_from_lds<PF_NQ>(PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), qf, my_kb, lo, hi, scale, sm,   \
                                         acc);                                                                   \
         }                                                                                                       \
         PF_STORE(NEXT, (KB) + STEP_KEYS, (STAGE) ^ 1);                                                          \
         __syncthreads();                                                                                        \
     } while (0)
-            PF_FETCH(regs_a, w_first);
-            PF_FETCH(regs_b, w_first + STEP_KEYS);
-            PF_STORE(regs_a, w_first, 0);
+            // steps past the last tile (to fill a group of AHEAD) load the last tile again, compute and store
+            // nothing and keep the barriers in step
+#pragma unroll
+            for (int j = 0; j < AHEAD; ++j) PF_FETCH(regs[j], w_first + j * STEP_KEYS);
+            PF_STORE(regs[0], w_first, 0);
             __syncthreads();
-            for (int kb = w_first; kb <= w_last; kb += 2 * STEP_KEYS) {
-                PF_STEP(regs_a, regs_b, kb, 0);
-                if (kb + STEP_KEYS <= w_last) PF_STEP(regs_b, regs_a, kb + STEP_KEYS, 1);
+            for (int kb = w_first; kb <= w_last; kb += AHEAD * STEP_KEYS) {
+#pragma unroll
+                for (int j = 0; j < AHEAD; ++j)
+                    PF_STEP(regs[j], regs[(j + 1) % AHEAD], kb + j * STEP_KEYS, j & 1);
             }
 #undef PF_STEP
 #undef PF_STORE
@@ -664,9 +736,10 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
             const int range_hi = first_pos + row_last;
             const int range_lo = window > 0 ? max(0, first_pos + row0 - window + 1) : 0;
             attend_range<PF_NQ>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, range_lo, range_hi, lo, hi, scale,
-                                m, l, acc);
+                                sm, acc);
         }
     }
+    sm.finish_sums();
 
     if constexpr (KSPLIT == 2) {
         // The waves of the second part hand (m, l, acc) to the waves of the first through LDS (the tiles are
@@ -677,8 +750,8 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
 #pragma unroll
             for (int n = 0; n < PF_NQ; ++n) {
                 float* b = box + n * (DBLOCKS * 4 + 2);
-                b[0] = m[n];
-                b[1] = l[n];
+                b[0] = sm.m[n];
+                b[1] = sm.l[n];
 #pragma unroll
                 for (int db = 0; db < DBLOCKS; ++db)
 #pragma unroll
@@ -690,10 +763,10 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
 #pragma unroll
         for (int n = 0; n < PF_NQ; ++n) {
             const float* b = box + n * (DBLOCKS * 4 + 2);
-            const float m_other = b[0], m_new = fmaxf(m[n], m_other);
+            const float m_other = b[0], m_new = fmaxf(sm.m[n], m_other);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float w_mine = fast_exp2(m[n] - m_use), w_other = fast_exp2(m_other - m_use);
-            l[n] = l[n] * w_mine + b[1] * w_other;
+            const float w_mine = fast_exp2(sm.m[n] - m_use), w_other = fast_exp2(m_other - m_use);
+            sm.l[n] = sm.l[n] * w_mine + b[1] * w_other;
 #pragma unroll
             for (int db = 0; db < DBLOCKS; ++db)
 #pragma unroll
@@ -706,7 +779,7 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     for (int n = 0; n < PF_NQ; ++n) {
         const int row = row0 + n * 16 + r;
         if (row >= q_len) continue;
-        const float inv = 1.f / l[n];
+        const float inv = 1.f / sm.l[n];
         bf16_t* dst = out + ((size_t)(q_begin + row) * n_heads + head) * HD;
 #pragma unroll
         for (int db = 0; db < DBLOCKS; ++db) {
@@ -721,6 +794,18 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
 // ---------------------------------------------------------------------------------------------------
 // entry points
 // ---------------------------------------------------------------------------------------------------
+// Compute units of the current device (asked once per device).
+static int compute_units() {
+    static int known[64];
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+    if (!known[device]) {
+        int n = 0;
+        known[device] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && n > 0) ? n : 256;
+    }
+    return known[device];
+}
+
 static int log2_exact(int v) {
     int l = 0;
     while ((1 << l) < v) ++l;
@@ -809,16 +894,17 @@ SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_p
     if constexpr (HD > 128) {
         return launch_prefill<1, PF_ROWS / 16, 1>(n_tiles, ARGS);
     } else {
-        // Measured at 24 heads of 128 : the split shape is the fastest while all its
-        // workgroups are on the chip at once (prompts or portions up to about 1,024 tokens), the 8-wave shape
-        // of 128 tokens (two tiles of keys a step) up to about 2,048, the wide shape (one tile a step) beyond,
-        // and from about 12,000 tokens on 8 waves of 32 tokens (256 tokens a workgroup, two tiles a step: a tile
-        // staged in LDS then serves twice as many tokens; 6 % faster at 16,384 and 32,768 tokens, not below).
-        const long long wide_groups = (long long)n_tiles * n_heads;
-        if (PF_USE_LDS && n_tiles_split > 0 && wide_groups <= 224)
+        // Which shape is the fastest follows the number of workgroups per compute unit (measured at 24 heads of 128
+        // on 256 compute units): the split shape while all its workgroups are on the chip at once (under 7/8 of a
+        // wide workgroup per compute unit: prompts or portions up to about 1,024 tokens), the 8-wave shape of 128
+        // tokens (two tiles of keys a step) up to 15/8 (about 2,048 tokens), the wide shape (one tile a step)
+        // beyond, and from 75/8 on (about 12,000 tokens) 8 waves of 32 tokens (256 tokens a workgroup, two tiles a
+        // step: a tile staged in LDS then serves twice as many tokens).
+        const long long wide_groups = (long long)n_tiles * n_heads, cus = compute_units();
+        if (PF_USE_LDS && n_tiles_split > 0 && wide_groups * 8 <= cus * 7)
             return launch_prefill<1, 2 * PF_ROWS_SPLIT / 16, 2>(n_tiles_split, ARGS);
-        if (wide_groups <= 480) return launch_prefill<1, PF_ROWS / 16, 1, PF_USE_LDS ? 2 : 1>(n_tiles, ARGS);
-        if (PF_USE_LDS && n_tiles_long > 0 && wide_groups >= 2400)
+        if (wide_groups * 8 <= cus * 15) return launch_prefill<1, PF_ROWS / 16, 1, PF_USE_LDS ? 2 : 1>(n_tiles, ARGS);
+        if (PF_USE_LDS && n_tiles_long > 0 && wide_groups * 8 >= cus * 75)
             return launch_prefill<2, PF_ROWS_LONG / 32, 1, 2>(n_tiles_long, ARGS);
         return launch_prefill<2, PF_ROWS / 32, 1>(n_tiles, ARGS);
     }

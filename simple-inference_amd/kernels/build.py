@@ -51,6 +51,17 @@ LINK_FLAGS: Dict[str, Sequence[str]] = {
     "blas": ("-L/opt/rocm/lib", "-lhipblaslt"),
 }
 
+# compiler flags of the libraries built from one source, beside HIPCC_FLAGS
+SOURCE_FLAGS: Dict[str, Sequence[str]] = {
+    # scores are never NaN (masked ones are -inf): a maximum then needs no quieting of signalling NaNs first, which
+    # costs an instruction per operand in the softmax of every tile
+    "attention_mfma.hip": ("-fno-honor-nans",),
+}
+
+
+def _source_flags(sources: Sequence[str]) -> list:
+    return [flag for src in sources for flag in SOURCE_FLAGS.get(Path(src).name, ())]
+
 
 class KernelBuildError(RuntimeError):
     pass
@@ -78,12 +89,12 @@ def _headers_of(sources: Iterable[Path]) -> list:
     return [found[name] for name in sorted(found)]
 
 
-def _digest(sources: Iterable[Path], defines: Sequence[str], link: Sequence[str] = ()) -> str:
+def _digest(sources: Sequence[Path], defines: Sequence[str], link: Sequence[str] = ()) -> str:
     h = hashlib.sha256()
     for path in list(sources) + _headers_of(sources):
         h.update(path.name.encode())
         h.update(path.read_bytes())
-    h.update(" ".join(list(HIPCC_FLAGS) + list(defines) + list(link)).encode())
+    h.update(" ".join(list(HIPCC_FLAGS) + _source_flags([p.name for p in sources]) + list(defines) + list(link)).encode())
     return h.hexdigest()[:12]
 
 
@@ -117,7 +128,7 @@ def compile_library(name: str, sources: Sequence[str], defines: Sequence[str] = 
     hipcc = find_hipcc()
     out.parent.mkdir(parents=True, exist_ok=True)
     tmp = out.with_suffix(f".tmp{os.getpid()}.so")
-    cmd = [hipcc, *HIPCC_FLAGS, *[f"-D{d}" for d in defines], f"-I{CSRC}",
+    cmd = [hipcc, *HIPCC_FLAGS, *_source_flags(sources), *[f"-D{d}" for d in defines], f"-I{CSRC}",
            *[str(CSRC / s) for s in sources], "-o", str(tmp), *LINK_FLAGS.get(name, ())]
     if verbose:
         print(f"[simple-inference_amd] compiling {name} ({', '.join(sources)}) for {ARCH} ...",
