@@ -214,13 +214,42 @@ def run_stream(preset_name, requests, max_running, max_seq_len, prefix_cache, ar
         return {f"p{q}": round(v[min(len(v) - 1, int(len(v) * q / 100))] * 1e3, 2) for q in (50, 90, 99)}
     ttft = [first[i] for i in by_id]                       # every request is queued at time 0
     tpot = [(last[i] - first[i]) / (len(by_id[i].generated) - 1) for i in by_id if len(by_id[i].generated) > 1]
+    check = stream_check(engine, [(list(h.prompt_tokens), list(h.generated)) for h in handles])
     out = {"seconds": round(sec, 3), "steps": engine.stats["steps"], "prompt_tokens": sum(len(p) for p, _ in requests),
            "prefill_tokens_run": engine.stats["prefill_tokens"], "generated_tokens": engine.stats["decode_tokens"] + len(requests),
            "generated_tok_s": round(sum(n for _, n in requests) / sec, 1),
-           "ttft_ms": percentiles(ttft), "tpot_ms": percentiles(tpot)}
+           "ttft_ms": percentiles(ttft), "tpot_ms": percentiles(tpot), "check": check}
     del engine
     torch.cuda.empty_cache()
     return out
+
+
+def stream_check(engine, finished, sample=4, last=8):
+    """Were the stream's tokens the right ones?  A few of its requests are run again alone, whole (prompt and what
+    the stream generated for it, in one step), and the stream's last tokens are compared with what that run would
+    choose at the same places: equal, or tied with it within bfloat16 rounding (the stream met those tokens in
+    steps of other sizes, which the BLAS library multiplies in another order)."""
+    from simple_inference_amd.engine import StepEntry
+
+    engine.reset()
+    picks = sorted({(len(finished) - 1) * i // max(sample - 1, 1) for i in range(sample)})
+    same = close = total = 0
+    for n, i in enumerate(picks):
+        prompt, generated = finished[i]
+        k = min(last, len(generated))
+        tokens = prompt + generated[:-1]
+        places = [len(tokens) - k + j for j in range(k)]          # the places that chose the last k tokens
+        rid = 10 ** 6 + n
+        engine.cache.admit(rid)
+        logits = engine.runner.run([StepEntry(rid, tokens, places)]).float()
+        engine.cache.release(rid)
+        for row, token in zip(logits, generated[-k:]):
+            best = int(row.argmax())
+            total += 1
+            same += best == token
+            close += best == token or float(row[best] - row[token]) <= 2.5e-2 * float(row.abs().max())
+    assert close == total, f"{total - close} of {total} checked tokens are not what a solo run would choose"
+    return {"requests": len(picks), "tokens": total, "same_as_solo": same, "tied_within_rounding": close - same}
 
 
 def stream_workload(args):
