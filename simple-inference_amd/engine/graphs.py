@@ -92,7 +92,7 @@ class GraphedDecode:
         """A step can be replayed if every request brings one token and wants its logits.  (A prompt's portion of
         one token that is not its last brings one token too, but wants nothing: such a step runs eagerly.)"""
         return 0 < len(entries) <= self.buckets[-1] and all(
-            len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+            len(e.tokens) == 1 and list(e.want) == [0] and not e.extra for e in entries)
 
     def bucket_of(self, rows: int) -> int:
         return next(b for b in self.buckets if b >= rows)

@@ -30,6 +30,7 @@ class StepEntry:
     tokens: Sequence[int]            # its next tokens, in order
     want: Sequence[int] = field(default_factory=list)  # places among ``tokens`` whose logits are wanted
     token_from: Optional[int] = None  # the one token is row ``token_from`` of the step's ``device_tokens``; ``tokens`` holds a placeholder
+    extra: Optional[dict] = None     # further integers per token, by name (e.g. a second position axis): each len(tokens) long
 
 
 class StepRunner:
@@ -43,7 +44,12 @@ class StepRunner:
 
     def _check(self, entries: List[StepEntry]) -> None:
         seen = set()
+        extra_keys = {key for e in entries if e.extra for key in e.extra}
         for e in entries:
+            for key in extra_keys:
+                if e.extra is None or key not in e.extra or len(e.extra[key]) != len(e.tokens):
+                    raise ValueError(f"request {e.req}: per-token values {key!r} must be given for every request of "
+                                     f"the step, one per token")
             if e.req in seen:
                 raise ValueError(f"request {e.req} appears twice in one step")
             seen.add(e.req)
@@ -87,8 +93,9 @@ class StepRunner:
         n_rows = sum(len(e.want) for e in entries)
 
         n_moved = len(from_device)
+        extra_keys = sorted({key for e in seqs if e.extra for key in e.extra})
         sizes = [n_tokens, n_tokens, n_tokens, n_seqs + 1, n_seqs, n_seqs, max(n_rows, 1)] + \
-                [n_seqs * width] * n_groups + [n_moved, n_moved]
+                [n_seqs * width] * n_groups + [n_moved, n_moved] + [n_tokens] * len(extra_keys)
         offsets = np.concatenate([[0], np.cumsum(sizes)])
         host = np.empty(int(offsets[-1]), dtype=np.int32)
         tok, pos, sot, cu, kvl, slots, rows = (host[offsets[i]:offsets[i + 1]] for i in range(7))
@@ -123,6 +130,13 @@ class StepRunner:
             dst[:] = [first_token[e.req] for e in from_device]
             src[:] = [e.token_from for e in from_device]
 
+        for i, key in enumerate(extra_keys):
+            col = host[offsets[9 + n_groups + i]:offsets[10 + n_groups + i]]
+            t = 0
+            for e in seqs:
+                col[t:t + len(e.tokens)] = e.extra[key]
+                t += len(e.tokens)
+
         dev = torch.from_numpy(host).to(self.device)
         part = lambda i: dev[int(offsets[i]):int(offsets[i + 1])]
         if n_moved:
@@ -135,6 +149,7 @@ class StepRunner:
             n_decode_seqs=n_decode, q_lens=q_lens,
         )
         ctx.block_tables = [part(7 + g).view(n_seqs, width) for g in range(n_groups)]
+        ctx.extra = {key: part(9 + n_groups + i) for i, key in enumerate(extra_keys)}
         return ctx
 
     @torch.no_grad()

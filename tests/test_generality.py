@@ -625,3 +625,112 @@ def test_the_compiled_kernels_refuse_a_head_size_beyond_their_limit_at_build_tim
     from simple_inference_amd.kernels import HipKernels, KernelError
     with pytest.raises(KernelError, match="head size 272"):
         build_model(dict(TINY_A, head_dim=272), EngineConfig(device="cuda:0", dtype="bfloat16", max_seq_len=64), HipKernels())
+
+
+# ---- a position encoding with a second axis, brought by the step's entries ------------------------------------------
+class TwoAxisAngles:
+    """Half of the rotary pairs turn with the token's position, the other half with a second number per token that the
+    caller brings (``StepEntry.extra["column"]``), as encodings for grids of patches do.  The package's rotation
+    kernel takes one table row per token, so this encoding hands its mixer a table indexed by a *combined* index
+    and says how to form it; here the toy mixer below forms it."""
+
+    def __init__(self, params, env):
+        self.rotary_dim, self.columns, self.env = int(params["rotary_dim"]), int(params["columns"]), env
+
+    def weight_specs(self):
+        return {}
+
+    def bind(self, tensors):
+        pass
+
+    def angles(self, positions, columns):
+        quarter = self.rotary_dim // 4
+        freq = 1.0 / (100.0 ** (torch.arange(quarter, dtype=torch.float32) / quarter))
+        return torch.cat([positions.float()[:, None] * freq, columns.float()[:, None] * freq], dim=-1)   # [N, rotary/2]
+
+
+class TwoAxisMixer:
+    """out = W_o . rotate(W_q h) with the two-axis angles: no attention, so that the test is about the step's
+    metadata reaching a part, nothing else."""
+
+    def __init__(self, params, env):
+        self.hidden, self.env = int(params["hidden_size"]), env
+        self.position = TwoAxisAngles({"rotary_dim": self.hidden, "columns": 8}, env)
+
+    def weight_specs(self):
+        return {"q": TensorSpec((self.hidden, self.hidden)), "o": TensorSpec((self.hidden, self.hidden))}
+
+    def bind(self, tensors):
+        self.w = tensors
+
+    def cache_need(self):
+        return None
+
+    def state_need(self):
+        return None
+
+    def forward(self, h, ctx, cache):
+        k = self.env.kernels
+        q = k.linear(h, self.w["q"]).float()
+        ang = self.position.angles(ctx.positions.cpu(), ctx.extra["column"].cpu()).to(q.device)
+        half = self.hidden // 2
+        a, b = q[:, :half], q[:, half:]
+        rotated = torch.cat([a * ang.cos() - b * ang.sin(), b * ang.cos() + a * ang.sin()], dim=-1)
+        return k.linear(rotated.to(h.dtype), self.w["o"])
+
+
+def test_a_second_position_axis_reaches_a_part_through_the_step(tmp_path):
+    """Entries bring a number per token beside the token id; the step function lays it out with the batch
+    (sequences that bring one token first) and hands it to the parts as ``ctx.extra``."""
+    def plan(cfg):
+        from simple_inference_amd.parts import PartSpec as P
+        norm = lambda name: P("rmsnorm", {"size": H, "eps": 1e-5}, {"weight": name})
+        layer = LayerSpec(mixer=P("test_two_axis", {"hidden_size": H}, {"q": "q", "o": "o"}),
+                          feed_forward=P("swiglu", {"hidden_size": H, "intermediate_size": 48},
+                                         {"gate": "gate", "up": "up", "down": "down"}),
+                          mixer_norm=norm("n1"), feed_forward_norm=norm("n2"))
+        return ModelPlan(hidden_size=H, vocab_size=V,
+                         embedding=P("embedding", {"vocab_size": V, "hidden_size": H}, {"weight": "embed"}),
+                         layers=[layer], final_norm=norm("final"),
+                         head=P("head", {"vocab_size": V, "hidden_size": H, "tied": True}, {}))
+    register_mixer("test_two_axis", TwoAxisMixer, replace=True)
+    register_architecture("ToyTwoAxis", lambda d: d, plan, replace=True)
+    try:
+        import plain_llama as plain
+        runner, cache, weights = make("twins", {"architectures": ["ToyTwoAxis"]})
+        w = {k: v.double() for k, v in weights.items()}
+        g = torch.Generator().manual_seed(4)
+        seqs = {r: (torch.randint(0, V, (n,), generator=g).tolist(), torch.randint(0, 8, (n,), generator=g).tolist())
+                for r, n in ((1, 9), (2, 1), (3, 6))}
+
+        def reference(tokens, columns):
+            T = len(tokens)
+            x = w["embed"][tokens]
+            q = plain.rms_norm(x, w["n1"], 1e-5) @ w["q"].T
+            quarter = H // 4
+            freq = (1.0 / (100.0 ** (torch.arange(quarter, dtype=torch.float32) / quarter))).double()
+            ang = torch.cat([torch.arange(T).double()[:, None] * freq, torch.tensor(columns).double()[:, None] * freq], -1)
+            a, b = q[:, :H // 2], q[:, H // 2:]
+            x = x + torch.cat([a * ang.cos() - b * ang.sin(), b * ang.cos() + a * ang.sin()], -1) @ w["o"].T
+            x = x + plain.swiglu_mlp(plain.rms_norm(x, w["n2"], 1e-5), w["gate"], w["up"], w["down"])
+            return plain.rms_norm(x, w["final"], 1e-5) @ w["embed"].T
+
+        for r in seqs:
+            cache.admit(r)
+        # first step: a portion of 1, the single token of 2, a portion of 3 (the step sorts 2 to the front)
+        first = [StepEntry(1, seqs[1][0][:4], [0, 3], extra={"column": seqs[1][1][:4]}),
+                 StepEntry(2, seqs[2][0], [0], extra={"column": seqs[2][1]}),
+                 StepEntry(3, seqs[3][0][:5], [4], extra={"column": seqs[3][1][:5]})]
+        out = runner.run(first)
+        want = torch.stack([reference(*seqs[1])[0], reference(*seqs[1])[3], reference(*seqs[2])[0], reference(*seqs[3])[4]])
+        assert rel_err(out, want) <= 2e-5
+        second = [StepEntry(3, seqs[3][0][5:], [0], extra={"column": seqs[3][1][5:]}),
+                  StepEntry(1, seqs[1][0][4:], [4], extra={"column": seqs[1][1][4:]})]
+        out = runner.run(second)
+        assert rel_err(out, torch.stack([reference(*seqs[3])[5], reference(*seqs[1])[8]])) <= 2e-5
+        with pytest.raises(ValueError, match="column"):     # every entry of a step must bring it, or none
+            runner.run([StepEntry(2, [1], [0]), StepEntry(3, [2], [0], extra={"column": [1]})])
+        assert cache.lengths[2] == 1 and cache.lengths[3] == 6      # the refused step took nothing
+    finally:
+        unregister_architecture("ToyTwoAxis")
+        MIXERS.unregister("test_two_axis")
