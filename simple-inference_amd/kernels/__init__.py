@@ -41,6 +41,7 @@ _SIGNATURES = {
     "sia_sample_static_max_rows": [],
     "sia_gemm_skinny": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_gemm_skinny_max_rows": [],
+    "sia_gemm_skinny_residual_blocks": [_c_int],
     "sia_gemm_skinny_swiglu": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_ptr],
     "sia_gemm_skinny_rope": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
                              _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_ptr],
@@ -270,7 +271,7 @@ class HipKernels:
         N = w.shape[0]
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
             # up to 16 rows: this package's kernel, whose sums do not depend on the number of rows
-            if self.use_skinny_gemm and M <= self._skinny_rows and N % 16 == 0 and K % 64 == 0:
+            if self.use_skinny_gemm and M <= self._skinny_rows and K % 64 == 0:
                 y = torch.empty((M, N), dtype=torch.float32 if out_float32 else torch.bfloat16, device=x.device)
                 self._check(self.core.sia_gemm_skinny(_ptr(x), _ptr(w), _ptr(y), M, N, K, int(out_float32),
                                                       self._stream()), "gemm_skinny")
@@ -296,7 +297,7 @@ class HipKernels:
         M, K = x.shape
         two_i = w_gate_up.shape[0]
         if (self.use_skinny_gemm and x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
-                and M <= self._skinny_rows and two_i % 32 == 0 and K % 64 == 0 and w_gate_up.shape[1] == K):
+                and M <= self._skinny_rows and two_i % 2 == 0 and K % 64 == 0 and w_gate_up.shape[1] == K):
             rows, partials, n_partials, eps = self._scaled(x)
             self._want(rows, "gated linear input")
             y = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=rows.device)
@@ -312,7 +313,7 @@ class HipKernels:
         that follows has it computed by ``linear_into_residual``, which saves the norm's own kernel."""
         if (self.use_skinny_gemm and self.fuse_norms and isinstance(x, torch.Tensor) and x.dim() == 2 and w.dim() == 2
                 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] == w.shape[1]
-                and 0 < x.shape[0] <= self._skinny_rows and w.shape[0] % 16 == 0 and w.shape[1] % 64 == 0):
+                and 0 < x.shape[0] <= self._skinny_rows and w.shape[1] % 64 == 0):
             return PendingProduct(x, w, self)
         return self.linear(x, w)
 
@@ -327,11 +328,11 @@ class HipKernels:
         M, K = x.shape
         N = w.shape[0]
         if (w.shape[1] != K or tuple(residual.shape) != (M, N) or tuple(gain.shape) != (N,) or M > self._skinny_rows
-                or N % 16 or K % 64):
+                or K % 64):
             raise KernelError(f"product into the residual does not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, "
                               f"residual {tuple(residual.shape)}, gain {tuple(gain.shape)}")
         rows = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-        partials = torch.empty((N // 16, 16), dtype=torch.float32, device=x.device)
+        partials = torch.empty((self.core.sia_gemm_skinny_residual_blocks(N), 16), dtype=torch.float32, device=x.device)
         self._check(self.core.sia_gemm_skinny_residual(_ptr(x), _ptr(w), M, N, K, _ptr(residual), _ptr(gain),
                                                        _ptr(rows), _ptr(partials), self._stream()),
                     "gemm_skinny_residual")
@@ -423,7 +424,7 @@ class HipKernels:
         k and v columns are not to be read (for few rows one kernel does all three and never writes them)."""
         M, K = x.shape
         if (self.use_skinny_gemm and self.fuse_rope and n_kv_written and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
-                and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 32 == 0 and K % 64 == 0):
+                and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 2 == 0 and K % 64 == 0):
             x, partials, n_partials, norm_eps = self._scaled(x)
             self._want(x, "q/k/v input")
             self._want(w_qkv, "q/k/v weight")

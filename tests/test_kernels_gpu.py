@@ -121,7 +121,8 @@ def test_gemm_generic(hip, dtype, shape):
         torch.testing.assert_close(out.double(), ref, **tol(dtype))
 
 
-@pytest.mark.parametrize("shape", [(1, 48, 64), (8, 5120, 3072), (16, 3072, 8192), (3, 16, 320), (11, 1008, 1024)])
+@pytest.mark.parametrize("shape", [(1, 48, 64), (8, 5120, 3072), (16, 3072, 8192), (3, 16, 320), (11, 1008, 1024),
+                                   (7, 203, 192), (2, 1, 64), (9, 4099, 128), (16, 16384, 576)])
 def test_gemm_skinny(hip, shape):
     """bfloat16 products with few rows: this package's kernel against a float64 product and the library."""
     M, N, K = shape
@@ -143,7 +144,8 @@ def test_gemm_skinny(hip, shape):
     assert torch.equal(hip.linear(x[:1].contiguous(), w), out16[:1])
 
 
-@pytest.mark.parametrize("shape", [(1, 32, 64), (8, 8192, 3072), (16, 1008, 512), (5, 96, 320), (40, 128, 256)])
+@pytest.mark.parametrize("shape", [(1, 32, 64), (8, 8192, 3072), (16, 1008, 512), (5, 96, 320), (40, 128, 256),
+                                   (3, 1, 64), (12, 333, 192), (16, 14336, 256)])
 def test_gated_linear(hip, shape):
     """The product with the SwiGLU activation in its epilogue (few rows) or after it, against the twin."""
     M, inter, K = shape
@@ -230,7 +232,7 @@ def test_rope_kv_write_and_attention(hip, dtype, geom):
 @pytest.mark.parametrize("geom", [
     # heads, kv heads, head_dim, page_size, hidden, rows
     (24, 8, 128, 64, 3072, 8), (3, 1, 32, 8, 192, 16), (5, 5, 96, 16, 1088, 1), (2, 1, 256, 32, 64, 5),
-    (7, 7, 64, 4, 2048, 13),
+    (7, 7, 64, 4, 2048, 13), (5, 1, 48, 16, 320, 9), (32, 8, 64, 16, 2048, 4), (1, 1, 16, 2, 64, 3),
 ])
 def test_qkv_product_that_rotates_and_writes_the_pages(hip, geom):
     """Few rows: one kernel multiplies, rotates q and k and writes k and v into the pages.  Compared with the
@@ -286,6 +288,7 @@ def test_qkv_product_that_rotates_and_writes_the_pages(hip, geom):
 @pytest.mark.parametrize("shape", [
     # rows, hidden, inner (the K of the product into the residual), intermediate of the gated product after it
     (8, 3072, 8192, 8192), (1, 3072, 3072, 8192), (16, 192, 64, 96), (5, 5120, 1024, 5120), (13, 1088, 2048, 320),
+    (4, 4160, 128, 1001), (16, 4096, 14336, 1024),
 ])
 def test_norm_shared_out_between_the_products_around_it(hip, shape):
     """Few rows: the product before a norm adds into the residual and leaves gain * x and sums of squares; the product
@@ -314,7 +317,7 @@ def test_norm_shared_out_between_the_products_around_it(hip, shape):
     torch.testing.assert_close(res_fused.double(), want, rtol=0, atol=2 ** -6)
     # what it leaves for the product after it: gain * x rounded once, and the sums of squares
     assert torch.equal(scaled.rows, (res_fused * gain).to(torch.bfloat16))
-    assert tuple(scaled.partials.shape) == (hidden // 16, 16)
+    assert scaled.partials.shape[1] == 16 and hidden / 16 <= scaled.partials.shape[0] <= hidden / 8 + 4   # blocks of 8 to 16 columns
     sums = scaled.partials[:, :rows].double().sum(0)
     torch.testing.assert_close(sums, res_fused.double().pow(2).sum(-1), rtol=1e-5, atol=0)
     rs = torch.rsqrt(sums / hidden + eps)[:, None]
