@@ -17,6 +17,9 @@
 namespace {
 
 constexpr size_t WORKSPACE_BYTES = 32u << 20;
+constexpr int TRIED = 24;        // candidates of the library that are timed for a shape of few rows
+constexpr int TIMED_RUNS = 4;
+constexpr int TRY_OUT_ROWS = 256;  // up to here a product streams its weights once and the candidates differ widely
 
 struct Plan {
     hipblasLtMatmulDesc_t op = nullptr;
@@ -40,7 +43,10 @@ State* state_of_current_device() {
     return g_state[dev];
 }
 
-bool make_plan(State& st, Plan& p, int M, int N, int K, bool out_float) {
+// With `try_out` the library's candidates for the shape are run on the operands of the call that asks (whose
+// result the call itself then overwrites) and the fastest is kept; else its first candidate is taken.
+bool make_plan(State& st, Plan& p, int M, int N, int K, bool out_float, bool try_out, const void* X, const void* W,
+               void* Y, hipStream_t stream) {
     const hipDataType out_type = out_float ? HIP_R_32F : HIP_R_16BF;
     if (hipblasLtMatmulDescCreate(&p.op, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return false;
     const hipblasOperation_t trans = HIPBLAS_OP_T, none = HIPBLAS_OP_N;
@@ -55,14 +61,45 @@ bool make_plan(State& st, Plan& p, int M, int N, int K, bool out_float) {
     if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return false;
     const size_t limit = WORKSPACE_BYTES;
     hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit));
-    hipblasLtMatmulHeuristicResult_t found[1];
+    hipblasLtMatmulHeuristicResult_t found[TRIED];
     int n_found = 0;
+    const int wanted = try_out ? TRIED : 1;
     const hipblasStatus_t status =
-        hipblasLtMatmulAlgoGetHeuristic(st.handle, p.op, p.a, p.b, p.c, p.c, pref, 1, found, &n_found);
+        hipblasLtMatmulAlgoGetHeuristic(st.handle, p.op, p.a, p.b, p.c, p.c, pref, wanted, found, &n_found);
     hipblasLtMatmulPreferenceDestroy(pref);
-    if (status != HIPBLAS_STATUS_SUCCESS || n_found < 1 || found[0].workspaceSize > WORKSPACE_BYTES) return false;
-    p.algo = found[0].algo;
-    p.workspace = found[0].workspaceSize;
+    if (status != HIPBLAS_STATUS_SUCCESS || n_found < 1) return false;
+    int best = -1;
+    float best_ms = 0.f;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    const bool timed = try_out && n_found > 1 && hipEventCreate(&t0) == hipSuccess && hipEventCreate(&t1) == hipSuccess;
+    const float one = 1.f, zero = 0.f;
+    for (int i = 0; i < n_found; ++i) {
+        if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > WORKSPACE_BYTES) continue;
+        if (!timed) {
+            best = i;
+            break;
+        }
+        // the real operands, the real stream: one run to load the code, then the time of TIMED_RUNS
+        float ms = 0.f;
+        bool ran = true;
+        for (int run = 0; run <= TIMED_RUNS && ran; ++run) {
+            if (run == 1) hipEventRecord(t0, stream);
+            ran = hipblasLtMatmul(st.handle, p.op, &one, W, p.a, X, p.b, &zero, Y, p.c, Y, p.c, &found[i].algo,
+                                  st.workspace, WORKSPACE_BYTES, stream) == HIPBLAS_STATUS_SUCCESS;
+        }
+        if (!ran || hipEventRecord(t1, stream) != hipSuccess || hipEventSynchronize(t1) != hipSuccess ||
+            hipEventElapsedTime(&ms, t0, t1) != hipSuccess)
+            continue;
+        if (best < 0 || ms < best_ms) {
+            best = i;
+            best_ms = ms;
+        }
+    }
+    if (t0) hipEventDestroy(t0);
+    if (t1) hipEventDestroy(t1);
+    if (best < 0) return false;
+    p.algo = found[best].algo;
+    p.workspace = found[best].workspaceSize;
     p.ok = true;
     return true;
 }
@@ -101,7 +138,11 @@ SIA_EXPORT int sia_blas_mm(const void* X, const void* W, void* Y, int M, int N, 
     auto it = st->plans.find(key);
     if (it == st->plans.end()) {
         Plan p;
-        make_plan(*st, p, M, N, K, out_float != 0);
+        // candidates cannot be timed while the stream is being captured into a graph: shapes that a graph will hold
+        // are met in the eager runs before its capture
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        const bool eager = hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone;
+        make_plan(*st, p, M, N, K, out_float != 0, eager && M <= TRY_OUT_ROWS, X, W, Y, stream);
         it = st->plans.emplace(key, p).first;
     }
     const Plan& p = it->second;
