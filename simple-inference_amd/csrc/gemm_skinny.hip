@@ -26,7 +26,6 @@
 #include "common.h"
 
 #include <initializer_list>
-#include <type_traits>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -74,8 +73,7 @@ struct Epilogue {
     RowScale scale;
 };
 
-// RB: blocks of 16 rows of W per workgroup; WAVES: 8 or 16 waves that split K; DEPTH: chunks (of two steps) whose
-// loads a wave has in flight together.
+// RB: blocks of bh rows of W per workgroup; WAVES: 8 or 16 waves that split K.
 //   EPI_STORE:   row block rb holds bh rows of W and gives as many columns of Y (TOut)
 //   EPI_SWIGLU:  W = [gate; up] of N rows each; the first RB / 2 row blocks are gate rows, the others the up rows of
 //                the same columns: Y = silu(gate) * up, in float, rounded once
@@ -91,7 +89,7 @@ struct Epilogue {
 // the gate half and row u of the up half of W), or a pair of columns that the rotation mixes (EPI_ROPE: unit u is
 // column u % (head_dim / 2) of head u / (head_dim / 2) together with the column head_dim / 2 further).  A workgroup
 // owns UNIT_BLOCKS blocks of bh consecutive units from blockIdx.x * UNIT_BLOCKS * bh on.
-template <typename TOut, int RB, int WAVES, int DEPTH, int EPI, bool SCALED>
+template <typename TOut, int RB, int WAVES, int EPI, bool SCALED>
 __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                      const bf16_t* __restrict__ W,
                                                                      TOut* __restrict__ Y, int M, int N, int K,
@@ -155,74 +153,42 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
 
     // acc[j] belongs to share wave + j * WAVES.  This wave's t-th chunk is chunk wave + t * WAVES, of share
     // (wave + t * WAVES) % 16 = wave + (t % SPW) * WAVES, so it goes into accumulator t % SPW; the chunks are
-    // taken in order of t, which is each share's own order.  With DEPTH > 0 chunks come in groups of DEPTH (a
-    // multiple of SPW): while one group is multiplied the loads of the next are in flight, in registers of their own.
+    // taken in order of t, which is each share's own order.  (Loading a second group of chunks into registers of
+    // their own while the first is multiplied was measured and changes nothing: enough waves are in flight.)
     floatx4 acc[SPW][RB];
 #pragma unroll
     for (int j = 0; j < SPW; ++j)
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) acc[j][rb] = floatx4{0.f, 0.f, 0.f, 0.f};
-    struct Chunk {
-        bf16x8 a[2][RB][2], b[2][2];
-    };
-    // k is the same in all lanes of the wave (a scalar): a step outside K is skipped by a branch of the wave, not
-    // by a mask of lanes.  K is a multiple of 64, so a step is inside or outside as a whole.
-    auto load = [&](Chunk& c, int k, auto checked) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-            if (!checked.value || k + u * SK_STEP < K) {
-#pragma unroll
-                for (int rb = 0; rb < RB; ++rb) {
-                    c.a[u][rb][0] = ld8(w_row[rb] + k + u * SK_STEP);
-                    c.a[u][rb][1] = ld8(w_row[rb] + k + u * SK_STEP + 8);
-                }
-                c.b[u][0] = ld8(x_row + k + u * SK_STEP);
-                c.b[u][1] = ld8(x_row + k + u * SK_STEP + 8);
-            }
-    };
-    auto multiply = [&](const Chunk& c, int k, floatx4(&into)[RB], auto checked) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-            if (!checked.value || k + u * SK_STEP < K) {
-#pragma unroll
-                for (int rb = 0; rb < RB; ++rb) {
-                    into[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c.a[u][rb][0], c.b[u][0], into[rb], 0, 0, 0);
-                    into[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c.a[u][rb][1], c.b[u][1], into[rb], 0, 0, 0);
-                }
-            }
-    };
     constexpr int HOP = WAVES * SK_CHUNK;  // from one chunk of the wave to its next
-    constexpr std::true_type checked{};
-    constexpr std::false_type inside{};
-    if constexpr (DEPTH == 0) {  // one chunk at a time, for shapes whose chunk fills the registers
-        for (int k0 = wave * SK_CHUNK; k0 < K; k0 += SPW * HOP) {
+    for (int k0 = wave * SK_CHUNK; k0 < K; k0 += SPW * HOP) {
 #pragma unroll
-            for (int j = 0; j < SPW; ++j) {
-                Chunk c;
-                load(c, k0 + j * HOP, checked);
-                multiply(c, k0 + j * HOP, acc[j], checked);
-            }
+        for (int j = 0; j < SPW; ++j) {
+            // k is the same in all lanes of the wave (a scalar): a step outside K is skipped by a branch of the
+            // wave, not by a mask of lanes.  K is a multiple of 64, so a step is inside or outside as a whole.
+            const int k = k0 + j * HOP;
+            bf16x8 a[2][RB][2], b[2][2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                if (k + u * SK_STEP < K) {
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb) {
+                        a[u][rb][0] = ld8(w_row[rb] + k + u * SK_STEP);
+                        a[u][rb][1] = ld8(w_row[rb] + k + u * SK_STEP + 8);
+                    }
+                    b[u][0] = ld8(x_row + k + u * SK_STEP);
+                    b[u][1] = ld8(x_row + k + u * SK_STEP + 8);
+                }
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                if (k + u * SK_STEP < K) {
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb) {
+                        acc[j][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][rb][0], b[u][0], acc[j][rb], 0, 0, 0);
+                        acc[j][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][rb][1], b[u][1], acc[j][rb], 0, 0, 0);
+                    }
+                }
         }
-    } else {
-        static_assert(DEPTH % SPW == 0, "a group of chunks covers every share of the wave equally");
-        Chunk now[DEPTH ? DEPTH : 1], next[DEPTH ? DEPTH : 1];
-        auto round = [&](int k0, auto how) {
-#pragma unroll
-            for (int d = 0; d < DEPTH; ++d) load(next[d], k0 + (DEPTH + d) * HOP, how);
-#pragma unroll
-            for (int d = 0; d < DEPTH; ++d) multiply(now[d], k0 + d * HOP, acc[d % SPW], how);
-#pragma unroll
-            for (int d = 0; d < DEPTH; ++d) load(now[d], k0 + (2 * DEPTH + d) * HOP, how);
-#pragma unroll
-            for (int d = 0; d < DEPTH; ++d) multiply(next[d], k0 + (DEPTH + d) * HOP, acc[d % SPW], how);
-        };
-        int k0 = wave * SK_CHUNK;
-#pragma unroll
-        for (int d = 0; d < DEPTH; ++d) load(now[d], k0 + d * HOP, checked);
-        // while every chunk a round touches lies inside K the round has no branch, and each product waits for its
-        // own loads only; the rounds at the end check every step
-        for (; k0 + (3 * DEPTH - 1) * HOP + SK_CHUNK <= K; k0 += 2 * DEPTH * HOP) round(k0, inside);
-        for (; k0 < K; k0 += 2 * DEPTH * HOP) round(k0, checked);
     }
     // acc[j][rb][i] = share wave + j * WAVES of row m = r, column 4g + i of row block rb
 #pragma unroll
@@ -385,15 +351,15 @@ template <typename TOut, int EPI>
 static void launch_skinny(const bf16_t* X, const bf16_t* W, TOut* Y, int M, int N, int K, const Epilogue& ep,
                           hipStream_t stream) {
     const Cut cut = cheapest(N, 1, {4, 2, 1});
-#define LAUNCH(RB, WAVES, DEPTH)                                                                                 \
-    hipLaunchKernelGGL((gemm_skinny_kernel<TOut, RB, WAVES, DEPTH, EPI, false>), dim3(cut.grid),                  \
+#define LAUNCH(RB, WAVES)                                                                                 \
+    hipLaunchKernelGGL((gemm_skinny_kernel<TOut, RB, WAVES, EPI, false>), dim3(cut.grid),                  \
                        dim3(WAVES * SIA_WAVE), 0, stream, X, W, Y, M, N, K, cut.bh, ep)
     if (cut.unit_blocks == 4)
-        LAUNCH(4, 8, 0);
+        LAUNCH(4, 8);
     else if (cut.unit_blocks == 2)
-        LAUNCH(2, 16, 0);
+        LAUNCH(2, 16);
     else
-        LAUNCH(1, 8, 2);
+        LAUNCH(1, 8);
 #undef LAUNCH
 }
 
@@ -440,7 +406,7 @@ SIA_EXPORT int sia_gemm_skinny_swiglu(const void* X, const void* W, void* Y, int
     ep.scale = RowScale{partials, n_partials, eps};
     const Cut cut = cheapest(inter, 2, {2, 1});
 #define LAUNCH(RB, WAVES, SCALED)                                                                                  \
-    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, RB, WAVES, 0, EPI_SWIGLU, SCALED>), dim3(cut.grid),              \
+    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, RB, WAVES, EPI_SWIGLU, SCALED>), dim3(cut.grid),              \
                        dim3(WAVES * SIA_WAVE), 0, stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, inter, \
                        K, cut.bh, ep)
     if (cut.unit_blocks == 2 && partials)
@@ -475,18 +441,18 @@ SIA_EXPORT int sia_gemm_skinny_rope(const void* X, const void* W, void* Y, int M
                       table_width, n_heads, n_kv, head_dim, page_size};
     ep.scale = RowScale{partials, n_partials, eps};
     const Cut cut = cut_for(heads * (head_dim / 2), 1, 2);
-#define LAUNCH(WAVES, DEPTH, SCALED)                                                                              \
-    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 2, WAVES, DEPTH, EPI_ROPE, SCALED>), dim3(cut.grid),            \
+#define LAUNCH(WAVES, SCALED)                                                                              \
+    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 2, WAVES, EPI_ROPE, SCALED>), dim3(cut.grid),            \
                        dim3(WAVES * SIA_WAVE), 0, stream, (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K,  \
                        cut.bh, ep)
     if (K >= 1024 && partials)
-        LAUNCH(16, 0, true);
+        LAUNCH(16, true);
     else if (K >= 1024)
-        LAUNCH(16, 0, false);
+        LAUNCH(16, false);
     else if (partials)
-        LAUNCH(8, 0, true);
+        LAUNCH(8, true);
     else
-        LAUNCH(8, 0, false);
+        LAUNCH(8, false);
 #undef LAUNCH
     return SIA_LAUNCH_CHECK();
 }
