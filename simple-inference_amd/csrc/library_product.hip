@@ -28,9 +28,11 @@ struct Plan {
     hipblasLtMatmulAlgo_t algo;
     size_t workspace = 0;
     bool ok = false;
+    bool tried_out = false;  // the algorithm was chosen by timing the candidates
 };
 
 struct State {
+    bool try_out = false;  // shapes met now will recur: time the candidates
     hipblasLtHandle_t handle = nullptr;
     void* workspace = nullptr;
     std::unordered_map<uint64_t, Plan> plans;
@@ -46,6 +48,14 @@ State* state_of_current_device() {
 
 // With `try_out` the library's candidates for the shape are run on the operands of the call that asks (whose
 // result the call itself then overwrites) and the fastest is kept; else its first candidate is taken.
+void release(Plan& p) {
+    if (p.a) hipblasLtMatrixLayoutDestroy(p.a);
+    if (p.b) hipblasLtMatrixLayoutDestroy(p.b);
+    if (p.c) hipblasLtMatrixLayoutDestroy(p.c);
+    if (p.op) hipblasLtMatmulDescDestroy(p.op);
+    p = Plan{};
+}
+
 bool make_plan(State& st, Plan& p, int M, int N, int K, bool out_float, bool try_out, const void* X, const void* W,
                void* Y, hipStream_t stream) {
     const hipDataType out_type = out_float ? HIP_R_32F : HIP_R_16BF;
@@ -103,6 +113,7 @@ bool make_plan(State& st, Plan& p, int M, int N, int K, bool out_float, bool try
     p.algo = found[best].algo;
     p.workspace = found[best].workspaceSize;
     p.ok = true;
+    p.tried_out = timed;
     return true;
 }
 
@@ -128,6 +139,16 @@ SIA_EXPORT int sia_blas_init() {
     return 0;
 }
 
+// While on, every product of up to TRY_OUT_ROWS rows whose shape has not been tried out yet runs the library's
+// candidates on its own operands first (a few milliseconds, once per shape) and keeps the fastest.  For callers who
+// know that the shapes they are running will recur many times, such as the runs before a graph is captured.
+SIA_EXPORT int sia_blas_try_out(int on) {
+    State* st = state_of_current_device();
+    if (!st) return 1;
+    st->try_out = on != 0;
+    return 0;
+}
+
 // 0: launched.  Anything else: nothing was launched (not initialised, or the library has no algorithm for the
 // shape), and the caller takes another way.
 SIA_EXPORT int sia_blas_mm(const void* X, const void* W, void* Y, int M, int N, int K, int out_float,
@@ -137,15 +158,21 @@ SIA_EXPORT int sia_blas_mm(const void* X, const void* W, void* Y, int M, int N, 
     if (M <= 0 || N <= 0 || K <= 0) return 2;
     const uint64_t key = ((uint64_t)(uint32_t)M << 42) ^ ((uint64_t)(uint32_t)N << 21) ^ (uint64_t)(uint32_t)K ^
                          ((uint64_t)(out_float ? 1 : 0) << 63);
+    // Candidates are timed only while the caller says that the shapes it runs will recur, and never while the stream
+    // is being captured into a graph (a graph's shapes are met in the eager runs before its capture).
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    const bool try_out = st->try_out && M <= TRY_OUT_ROWS && hipStreamIsCapturing(stream, &capturing) == hipSuccess &&
+                         capturing == hipStreamCaptureStatusNone;
     auto it = st->plans.find(key);
-    if (it == st->plans.end()) {
+    if (it == st->plans.end() || (try_out && !it->second.tried_out)) {
         Plan p;
-        // candidates cannot be timed while the stream is being captured into a graph: shapes that a graph will hold
-        // are met in the eager runs before its capture
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        const bool eager = hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone;
-        make_plan(*st, p, M, N, K, out_float != 0, eager && M <= TRY_OUT_ROWS, X, W, Y, stream);
-        it = st->plans.emplace(key, p).first;
+        make_plan(*st, p, M, N, K, out_float != 0, try_out, X, W, Y, stream);
+        if (it != st->plans.end()) {
+            release(it->second);
+            it->second = p;
+        } else {
+            it = st->plans.emplace(key, p).first;
+        }
     }
     const Plan& p = it->second;
     if (!p.ok) return 3;

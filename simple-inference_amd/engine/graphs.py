@@ -19,6 +19,7 @@ torch's current stream, so they are captured with the library products between t
 
 from __future__ import annotations
 
+import contextlib
 import gc
 from typing import Dict, List
 
@@ -182,7 +183,9 @@ class GraphedDecode:
         model = self.runner.model
         side = torch.cuda.Stream(device=self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))
-        with torch.cuda.stream(side):
+        # what these runs launch is what every replay will launch: worth choosing library algorithms by measurement
+        settle = getattr(self.runner.kernels, "recurring_shapes", contextlib.nullcontext)
+        with torch.cuda.stream(side), settle():
             for _ in range(3):
                 model.forward(b.ctx, b.caches)
         torch.cuda.current_stream(self.device).wait_stream(side)

@@ -13,6 +13,7 @@ rows and the whole 32-bit path use this package's own kernels.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from typing import Optional
 
@@ -145,12 +146,29 @@ class HipKernels:
             lib.sia_blas_init.argtypes, lib.sia_blas_init.restype = [], ctypes.c_int
             lib.sia_blas_mm.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
             lib.sia_blas_mm.restype = ctypes.c_int
+            lib.sia_blas_try_out.argtypes, lib.sia_blas_try_out.restype = [_c_int], ctypes.c_int
             with torch.cuda.device(self.device):
                 if lib.sia_blas_init() != 0:
                     return None
             return lib
         except (build.KernelBuildError, OSError, AttributeError):
             return None
+
+    @contextlib.contextmanager
+    def recurring_shapes(self):
+        """Inside, the products that go to the BLAS library have the library's candidate algorithms timed on their
+        own operands when their shape is first met (few rows only), and the fastest kept.  For runs whose shapes will
+        recur many times: the eager runs before a graph is captured."""
+        if self.blas is None:
+            yield
+            return
+        with torch.cuda.device(self.device):
+            self.blas.sia_blas_try_out(1)
+        try:
+            yield
+        finally:
+            with torch.cuda.device(self.device):
+                self.blas.sia_blas_try_out(0)
 
     def _library_product(self, x, w, out_float32):
         """``x @ w^T`` for bfloat16 operands by the BLAS library, float accumulation."""

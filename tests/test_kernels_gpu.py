@@ -178,6 +178,24 @@ def test_library_product_called_directly(hip, shape):
         torch.testing.assert_close(wide.double(), ref, rtol=1e-2, atol=1e-2 * math.sqrt(K / 64))
 
 
+@pytest.mark.parametrize("shape", [(64, 3072, 3072), (33, 1008, 200), (256, 320, 512), (300, 128, 64)])
+def test_library_product_with_candidates_tried_out(hip, shape):
+    """Inside ``recurring_shapes`` the library's candidate algorithms are timed on the call's own operands and one is
+    kept: the product is right on that call and on those after it, inside and outside, also for a shape that had an
+    algorithm before."""
+    M, N, K = shape
+    assert hip.blas is not None
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=3), rnd(N, K, dtype=torch.bfloat16, seed=4)
+    ref = x.double() @ w.double().T
+    outs = [hip.linear(x, w)]
+    with hip.recurring_shapes():
+        outs += [hip.linear(x, w), hip.linear(x, w, out_float32=True)]
+    outs += [hip.linear(x, w)]
+    for out in outs:
+        torch.testing.assert_close(out.double(), ref, rtol=1e-2, atol=1e-2 * math.sqrt(K / 64))
+    assert torch.equal(outs[1], outs[3])   # the kept algorithm is used from then on
+
+
 def test_float32_product_has_no_reduced_precision(hip):
     """An operand bit below bfloat16 (8 bits) and tf32 (10 bits) resolution must reach the product."""
     K = 8
