@@ -336,13 +336,13 @@ static Cut cut_for(int units, int unit_blocks, int rows_per_unit) {
     return best;
 }
 
-// Of the cuts an epilogue has kernels for, the cheapest; of equals the one with more blocks per workgroup (fewer
-// workgroups fetch X).
+// Of the cuts an epilogue has kernels for, the cheapest; of equals the one with the higher blocks (fewer lanes that
+// repeat a row), then the one with more blocks per workgroup (fewer workgroups fetch X).
 static Cut cheapest(int units, int rows_per_unit, std::initializer_list<int> unit_blocks) {
     Cut best{0, 0, 0, 0};
     for (int ub : unit_blocks) {
         const Cut c = cut_for(units, ub, rows_per_unit);
-        if (!best.grid || c.cost < best.cost) best = c;
+        if (!best.grid || c.cost < best.cost || (c.cost == best.cost && c.bh > best.bh)) best = c;
     }
     return best;
 }
