@@ -228,7 +228,10 @@ def stream_check(engine, finished, sample=4, last=8):
     """Were the stream's tokens the right ones?  A few of its requests are run again alone, whole (prompt and what
     the stream generated for it, in one step), and the stream's last tokens are compared with what that run would
     choose at the same places: equal, or tied with it within bfloat16 rounding (the stream met those tokens in
-    steps of other sizes, which the BLAS library multiplies in another order)."""
+    steps of other sizes, which the BLAS library multiplies in another order).  Two logits count as tied if they
+    are no further apart than twice what the reference allows one logit of its fast path to be from its plain
+    one at full size (``benchmarks/bench_paged_cudagraph.py:236-264``: 0.15 + 0.05 |logit|); a token from a wrong
+    page or a wrong row would be several units away."""
     from simple_inference_amd.engine import StepEntry
 
     engine.reset()
@@ -247,7 +250,7 @@ def stream_check(engine, finished, sample=4, last=8):
             best = int(row.argmax())
             total += 1
             same += best == token
-            close += best == token or float(row[best] - row[token]) <= 2.5e-2 * float(row.abs().max())
+            close += best == token or float(row[best] - row[token]) <= 2 * (0.15 + 0.05 * abs(float(row[best])))
     assert close == total, f"{total - close} of {total} checked tokens are not what a solo run would choose"
     return {"requests": len(picks), "tokens": total, "same_as_solo": same, "tied_within_rounding": close - same}
 
@@ -312,8 +315,9 @@ def main(argv=None):
 
     dt, tok_s, gbs = decode_point(args.batch)
     line = {
-        "metric": "decode tok/s at batch 8; prefill tok/s at 2,048 tokens (3B, bf16)"
-                  if args.batch == 8 else f"decode tok/s at batch {args.batch}",
+        "metric": (f"decode tok/s at batch 8; prefill tok/s at {args.prefill_tokens:,} tokens "
+                   f"({args.preset.rsplit('-', 1)[-1].upper()}, {dt_name})")
+                  if args.batch == 8 and not args.no_prefill else f"decode tok/s at batch {args.batch}",
         "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dt_name, "data": "synthetic (seeded random weights N(0, 0.02) and uniform-random token ids)",
