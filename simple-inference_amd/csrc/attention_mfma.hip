@@ -333,15 +333,39 @@ __host__ __device__ inline int decode_splits(int n_tiles) {
     return s;
 }
 
+// out = sum_s w_s acc_s / sum_s w_s l_s over the splits of one (sequence, head), with w_s = 2^(m_s - max m) (the
+// maxima are kept in units of log2; a split without keys has m = -inf and weight 0).  One element: `at(s)` gives
+// split s's (acc, m, l).  Summed in split order with fused multiply-adds, the same wherever it is called from.
+template <typename At>
+__device__ __forceinline__ float merge_splits(int n_splits, float mx, At at) {
+    float o = 0.f, denom = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += 4) {  // four splits' loads in flight at a time
+        float acc[4], m[4], l[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) at(min(s0 + j, n_splits - 1), acc[j], m[j], l[j]);  // past the end: the last again, weight 0
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float w = s0 + j < n_splits ? fast_exp2(m[j] - mx) : 0.f;
+            denom = __builtin_fmaf(w, l[j], denom);
+            o = __builtin_fmaf(w, acc[j], o);
+        }
+    }
+    return o * (1.f / denom);
+}
+
+// Grid (kv heads, sequences, splits), or with `fold` (kv heads, sequences, 1): a workgroup then takes the splits of
+// its (sequence, kv head) one after the other, keeps their results in LDS and merges them itself, the way the
+// combine kernel does, bit for bit.  For steps of so many sequences that the splits are not needed to fill the
+// device: no partial results in memory and no second kernel.
 __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
-    bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window) {
-    extern __shared__ float lds[];  // [DEC_WAVES][group][HD + 2]
+    bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window, int max_splits, int fold) {
+    extern __shared__ float lds[];  // [DEC_WAVES][group][HD + 2], with fold then [max_splits][group][HD + 2]
     // splits are the slowest index of the grid: the workgroups that leave at once (splits a sequence does not
     // have) then come last, not interleaved with the others, which the chip deals out to its dies in turn
-    const int hk = blockIdx.x, seq = blockIdx.y, split = blockIdx.z, max_splits = gridDim.z;
+    const int hk = blockIdx.x, seq = blockIdx.y;
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     // The tiles that hold visible keys are dealt evenly, in order, to the n_splits * DEC_WAVES waves that
     // work for this (sequence, kv head): every wave gets a contiguous run, runs differ by one tile at most.
@@ -349,72 +373,100 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
     const int t_first = lo_all / TILE, n_tiles = pos / TILE - t_first + 1;
     const int n_splits = min(decode_splits(n_tiles), max_splits);
-    if (split >= n_splits) return;  // the whole workgroup: the grid is sized for the longest sequence there may be
+    if (!fold && (int)blockIdx.z >= n_splits) return;  // the whole workgroup: the grid is sized for the longest sequence there may be
     scale *= LOG2E;  // exponentials are taken as powers of two
     const int group = n_heads / n_kv;
     const int* table = block_table + (size_t)seq * table_width;
     bf16x8 qf[1][KSTEPS];
     load_q(qf[0], r < group ? q + (size_t)seq * q_row_stride + (hk * group + r) * HD : nullptr, g);
-    const int n_waves = n_splits * DEC_WAVES, wi = split * DEC_WAVES + wave;
-    const int my_first = t_first + (int)(((long long)wi * n_tiles) / n_waves);
-    const int my_end = t_first + (int)(((long long)(wi + 1) * n_tiles) / n_waves);
-
-    Softmax<1> sm;
-    sm.start();
-    floatx4 acc[1][DBLOCKS];
-#pragma unroll
-    for (int db = 0; db < DBLOCKS; ++db) acc[0][db] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    if (my_first < my_end) {  // wave-uniform
-        const int w_lo = max(lo_all, my_first * TILE), w_hi = min(pos, my_end * TILE - 1);
-        const int lo[1] = {r < group ? w_lo : 1}, hi[1] = {r < group ? w_hi : 0};
-        attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, sm, acc);
-    }
-    sm.finish_sums();
-
+    const int n_waves = n_splits * DEC_WAVES;
     constexpr int ROW = HD + 2;
-    if (r < group) {
-        float* mine = lds + (size_t)(wave * group + r) * ROW;
-        if (g == 0) {
-            mine[HD] = sm.m[0];
-            mine[HD + 1] = sm.l[0];
+    float* const kept = lds + (size_t)DEC_WAVES * group * ROW;  // with fold: the splits' results
+
+    const int split_first = fold ? 0 : blockIdx.z, split_end = fold ? n_splits : blockIdx.z + 1;
+    for (int split = split_first; split < split_end; ++split) {
+        const int wi = split * DEC_WAVES + wave;
+        const int my_first = t_first + (int)(((long long)wi * n_tiles) / n_waves);
+        const int my_end = t_first + (int)(((long long)(wi + 1) * n_tiles) / n_waves);
+
+        Softmax<1> sm;
+        sm.start();
+        floatx4 acc[1][DBLOCKS];
+#pragma unroll
+        for (int db = 0; db < DBLOCKS; ++db) acc[0][db] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+        if (my_first < my_end) {  // wave-uniform
+            const int w_lo = max(lo_all, my_first * TILE), w_hi = min(pos, my_end * TILE - 1);
+            const int lo[1] = {r < group ? w_lo : 1}, hi[1] = {r < group ? w_hi : 0};
+            attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, sm, acc);
         }
+        sm.finish_sums();
+
+        if (split != split_first) __syncthreads();  // the split before has been read out of the waves' rows
+        if (r < group) {
+            float* mine = lds + (size_t)(wave * group + r) * ROW;
+            if (g == 0) {
+                mine[HD] = sm.m[0];
+                mine[HD + 1] = sm.l[0];
+            }
 #pragma unroll
-        for (int db = 0; db < DBLOCKS; ++db)
+            for (int db = 0; db < DBLOCKS; ++db)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) mine[db * 16 + g * 4 + i] = acc[0][db][i];
+                for (int i = 0; i < 4; ++i) mine[db * 16 + g * 4 + i] = acc[0][db][i];
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < group * HD; idx += DEC_WAVES * SIA_WAVE) {
+            const int c = idx / HD, d = idx % HD;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, lds[(size_t)(w * group + c) * ROW + HD]);
+            const float mx_use = (mx == -INFINITY) ? 0.f : mx;  // no wave had a key: all weights 0, the split counts for nothing
+            float o = 0.f, lsum = 0.f;
+#pragma unroll
+            for (int w = 0; w < DEC_WAVES; ++w) {
+                const float* row = lds + (size_t)(w * group + c) * ROW;
+                const float wgt = fast_exp2(row[HD] - mx_use);  // a wave without keys has m = -inf: weight 0
+                o += wgt * row[d];
+                lsum += wgt * row[HD + 1];
+            }
+            if (n_splits == 1) {  // nothing to combine with: this is the result
+                out[((size_t)cu_q[seq] * n_heads + hk * group + c) * HD + d] = float_to_bf16(o * (1.f / lsum));
+                continue;
+            }
+            if (fold) {
+                float* row = kept + (size_t)(split * group + c) * ROW;
+                row[d] = o;
+                if (d == 0) {
+                    row[HD] = mx;
+                    row[HD + 1] = lsum;
+                }
+                continue;
+            }
+            const size_t slot = ((size_t)seq * n_heads + hk * group + c) * max_splits + split;
+            ws_acc[slot * HD + d] = o;
+            if (d == 0) {
+                ws_ml[slot * 2] = mx;
+                ws_ml[slot * 2 + 1] = lsum;
+            }
+        }
     }
+    if (!fold || n_splits == 1) return;
     __syncthreads();
     for (int idx = threadIdx.x; idx < group * HD; idx += DEC_WAVES * SIA_WAVE) {
         const int c = idx / HD, d = idx % HD;
         float mx = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, lds[(size_t)(w * group + c) * ROW + HD]);
-        const float mx_use = (mx == -INFINITY) ? 0.f : mx;  // no wave had a key: all weights 0, the split counts for nothing
-        float o = 0.f, lsum = 0.f;
-#pragma unroll
-        for (int w = 0; w < DEC_WAVES; ++w) {
-            const float* row = lds + (size_t)(w * group + c) * ROW;
-            const float wgt = fast_exp2(row[HD] - mx_use);  // a wave without keys has m = -inf: weight 0
-            o += wgt * row[d];
-            lsum += wgt * row[HD + 1];
-        }
-        if (n_splits == 1) {  // nothing to combine with: this is the result
-            out[((size_t)cu_q[seq] * n_heads + hk * group + c) * HD + d] = float_to_bf16(o * (1.f / lsum));
-            continue;
-        }
-        const size_t slot = ((size_t)seq * n_heads + hk * group + c) * max_splits + split;
-        ws_acc[slot * HD + d] = o;
-        if (d == 0) {
-            ws_ml[slot * 2] = mx;
-            ws_ml[slot * 2 + 1] = lsum;
-        }
+        for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, kept[(size_t)(s * group + c) * ROW + HD]);
+        const float o = merge_splits(n_splits, mx, [&](int s, float& acc, float& m, float& l) {
+            const float* row = kept + (size_t)(s * group + c) * ROW;
+            acc = row[d];
+            m = row[HD];
+            l = row[HD + 1];
+        });
+        out[((size_t)cu_q[seq] * n_heads + hk * group + c) * HD + d] = float_to_bf16(o);
     }
 }
 
-// Combines the splits of each (sequence, head): out = sum_s w_s acc_s / sum_s w_s l_s with
-// w_s = 2^(m_s - max m) (the maxima are kept in units of log2; a split without keys has m = -inf and weight
-// 0), summed in split order, eight splits' loads in flight at a time.
+// Combines the splits of each (sequence, head) that workgroups of their own left in the workspaces.
 __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
     const float* __restrict__ ws_acc, const float* __restrict__ ws_ml, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int max_splits, int window) {
@@ -423,46 +475,16 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
     const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
     const int n_splits = min(decode_splits(pos / TILE - lo_all / TILE + 1), max_splits);
     if (n_splits == 1) return;  // its one workgroup wrote the result itself
-    const int first = 0, last = n_splits - 1;
     const size_t base = ((size_t)seq * n_heads + head) * max_splits;
     float mx = -INFINITY;
-    for (int s0 = first; s0 <= last; s0 += SIA_WAVE) {
-        const int s = s0 + lane;
-        mx = fmaxf(mx, s <= last ? ws_ml[(base + s) * 2] : -INFINITY);
-    }
-    mx = wave_max(mx);
-    float denom = 0.f;
-    constexpr int DD = (HD + SIA_WAVE - 1) / SIA_WAVE;
-    float o[DD];
-#pragma unroll
-    for (int dd = 0; dd < DD; ++dd) o[dd] = 0.f;
-    for (int s0 = first; s0 <= last; s0 += 8) {
-        float w[8], part[8][DD];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int s = min(s0 + j, last);  // a clamped slot is read again with weight 0
-            const bool live = s0 + j <= last;
-            w[j] = live ? fast_exp2(ws_ml[(base + s) * 2] - mx) : 0.f;
-            denom += live ? w[j] * ws_ml[(base + s) * 2 + 1] : 0.f;
-#pragma unroll
-            for (int dd = 0; dd < DD; ++dd) {
-                const int d = lane + dd * SIA_WAVE;
-                part[j][dd] = d < HD ? ws_acc[(base + s) * HD + d] : 0.f;
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-#pragma unroll
-            for (int dd = 0; dd < DD; ++dd) o[dd] += w[j] * part[j][dd];
-    }
-    const int token = cu_q[seq];
-    bf16_t* dst = out + ((size_t)token * n_heads + head) * HD;
-    const float inv = 1.f / denom;
-#pragma unroll
-    for (int dd = 0; dd < DD; ++dd) {
-        const int d = lane + dd * SIA_WAVE;
-        if (d < HD) dst[d] = float_to_bf16(o[dd] * inv);
-    }
+    for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, ws_ml[(base + s) * 2]);
+    bf16_t* dst = out + ((size_t)cu_q[seq] * n_heads + head) * HD;
+    for (int d = lane; d < HD; d += SIA_WAVE)
+        dst[d] = float_to_bf16(merge_splits(n_splits, mx, [&](int s, float& acc, float& m, float& l) {
+            acc = ws_acc[(base + s) * HD + d];
+            m = ws_ml[(base + s) * 2];
+            l = ws_ml[(base + s) * 2 + 1];
+        }));
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -839,13 +861,32 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
         n_splits > DEC_MAX_SPLITS || n_kv > 65535 || n_seqs > 65535 || q_row_stride % 8 || table_width <= 0 ||
         (n_splits > 1 && (!ws_acc || !ws_ml)))
         return SIA_BAD_ARGUMENT;
-    const size_t lds_bytes = (size_t)DEC_WAVES * (n_heads / n_kv) * (HD + 2) * sizeof(float);
+    const size_t row_bytes = (size_t)(n_heads / n_kv) * (HD + 2) * sizeof(float);
+    size_t lds_bytes = DEC_WAVES * row_bytes;
     if (lds_bytes > 64 * 1024) return SIA_BAD_ARGUMENT;
-    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_kv, n_seqs, n_splits), dim3(DEC_WAVES * SIA_WAVE), lds_bytes,
-                       stream, (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
-                       block_table, table_width, cu_q, kv_len, ws_acc, ws_ml, (bf16_t*)out, n_heads, n_kv, ps_log2,
-                       scale, window);
-    if (n_splits > 1)
+    // With two workgroups or more for every compute unit without them, the splits of a (sequence, kv head) are
+    // taken by one workgroup in turn (if their results fit into its LDS): the same numbers, one kernel.
+    const bool fold = n_splits > 1 && (long long)n_kv * n_seqs >= 2ll * compute_units() &&
+                      lds_bytes + n_splits * row_bytes <= 64 * 1024;
+    if (fold) {
+        lds_bytes += n_splits * row_bytes;
+        if (lds_bytes > 48 * 1024) {  // beyond the default limit of dynamic LDS
+            static bool allowed[64];
+            int device = 0;
+            if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return SIA_BAD_ARGUMENT;
+            if (!allowed[device]) {
+                const hipError_t e = hipFuncSetAttribute((const void*)attn_decode_kernel,
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+                if (e != hipSuccess) return (int)e;
+                allowed[device] = true;
+            }
+        }
+    }
+    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_kv, n_seqs, fold ? 1 : n_splits), dim3(DEC_WAVES * SIA_WAVE),
+                       lds_bytes, stream, (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages,
+                       (const bf16_t*)v_pages, block_table, table_width, cu_q, kv_len, ws_acc, ws_ml, (bf16_t*)out,
+                       n_heads, n_kv, ps_log2, scale, window, n_splits, fold ? 1 : 0);
+    if (n_splits > 1 && !fold)
         hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_heads, n_seqs), dim3(SIA_WAVE), 0, stream, ws_acc,
                            ws_ml, cu_q, kv_len, (bf16_t*)out, n_heads, n_splits, window);
     return SIA_LAUNCH_CHECK();

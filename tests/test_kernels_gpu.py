@@ -437,11 +437,16 @@ def test_decode_attention_of_a_sequence_does_not_depend_on_its_batch(hip, geom):
     torch.testing.assert_close(torch.stack([together[i] for i in everyone]).float(), ref.float(), **tol(dtype))
     bounded = run(everyone, bound=16384)
     many = run(everyone, repeat=6)                    # 72 sequences: more workgroups than compute units
+    # so many that one workgroup takes all the splits of a (sequence, kv head) in turn and merges them itself
+    crowd = run(everyone, repeat=-(-600 // (n_kv * len(everyone))))
+    crowd_bounded = run(everyone, bound=16384, repeat=-(-600 // (n_kv * len(everyone))))
     for i in everyone:
         alone = run([i])[i]
         assert torch.equal(alone, together[i]), kv_lens[i]
         assert torch.equal(alone, bounded[i]), kv_lens[i]
         assert torch.equal(alone, many[i]), kv_lens[i]
+        assert torch.equal(alone, crowd[i]), kv_lens[i]
+        assert torch.equal(alone, crowd_bounded[i]), kv_lens[i]
     pair = run([3, 9])
     assert torch.equal(pair[3], together[3]) and torch.equal(pair[9], together[9])
 
