@@ -69,7 +69,8 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, int row_stride, co
                                          const float* __restrict__ sin_table, const int* __restrict__ positions,
                                          const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                          int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                         int n_heads, int n_kv, int head_dim, int rotary_dim, int page_size) {
+                                         int n_heads, int n_kv, int head_dim, int rotary_dim, int page_size,
+                                         int v_group) {
     const int n = blockIdx.x;
     const int pos = positions[n];
     const int half = rotary_dim / 2, pairs = half / 8, plain = (head_dim - rotary_dim) / 8, pieces = head_dim / 8;
@@ -81,7 +82,8 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, int row_stride, co
         page = block_table[(size_t)seq_of_token[n] * table_width + pos / page_size];
         off = pos % page_size;
     }
-    const int items_q = n_heads * pairs, items_kr = n_kv * pairs, items_kp = n_kv * plain, items_v = n_kv * pieces;
+    const int items_q = n_heads * pairs, items_kr = n_kv * pairs, items_kp = n_kv * plain;
+    const int items_v = v_group ? 0 : n_kv * pieces;
     for (int item = threadIdx.x; item < items_q + items_kr + items_kp + items_v; item += blockDim.x) {
         if (item < items_q + items_kr) {  // a rotated pair of q (in place) or of k (into the page)
             const bool is_q = item < items_q;
@@ -117,7 +119,7 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, int row_stride, co
             Vec8<T> v;
             v.load(row + (n_heads + h) * head_dim + j);
             if (page >= 0) v.store(k_pages + (((size_t)page * n_kv + h) * page_size + off) * head_dim + j);
-        } else if (page >= 0) {  // v: 8 dims, each to its own row of the page (positions are innermost there)
+        } else if (page >= 0 && v_group == 0) {  // v: 8 dims, each to its own row of the page (positions are innermost there)
             const int it = item - items_q - items_kr - items_kp;
             const int h = it / pieces, j = (it % pieces) * 8;
             const T* x = row + (n_heads + n_kv + h) * head_dim + j;
@@ -125,6 +127,35 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, int row_stride, co
 #pragma unroll
             for (int i = 0; i < 8; ++i) dst[(size_t)i * page_size] = x[i];
         }
+    }
+    if (v_group == 0 || page < 0) return;
+    // v, for pages of 8 or 16 positions and more.  Positions are innermost in a page, so where v_group consecutive
+    // tokens of one sequence fill an aligned run of a page, their workgroups share the work by dims, not by tokens:
+    // each takes a slice of the (head, dim) rows and writes all the group's positions of a row at once (16 or 32
+    // contiguous bytes in bfloat16, neighbouring lanes neighbouring rows), instead of one element per token and row.
+    const int seq = seq_of_token[n];
+    const int place = off % v_group, first = n - place, rows = n_kv * head_dim;
+    const bool whole = first >= 0 && first + v_group <= (int)gridDim.x && seq_of_token[first] == seq &&
+                       seq_of_token[first + v_group - 1] == seq && positions[first] == pos - place &&
+                       positions[first + v_group - 1] == pos - place + v_group - 1;
+    if (!whole) {  // an incomplete group: every token writes its own values
+        const T* x = row + (n_heads + n_kv) * head_dim;
+        for (int i = threadIdx.x; i < rows; i += blockDim.x)
+            v_pages[((size_t)page * rows + i) * page_size + off] = x[i];
+        return;
+    }
+    constexpr int V_MAX = 16;
+    const int slice = (rows + v_group - 1) / v_group;
+    const T* x0 = qkv + (size_t)first * row_stride + (n_heads + n_kv) * head_dim;
+    for (int i = place * slice + threadIdx.x; i < min(rows, (place + 1) * slice); i += blockDim.x) {
+        __attribute__((aligned(16))) T vals[V_MAX];
+#pragma unroll
+        for (int j = 0; j < V_MAX; ++j) vals[j] = j < v_group ? x0[(size_t)j * row_stride + i] : T(0);
+        T* dst = v_pages + ((size_t)page * rows + i) * page_size + (off - place);
+        constexpr int PER = 16 / sizeof(T);  // elements of a 16-byte store
+#pragma unroll
+        for (int j = 0; j < V_MAX; j += PER)
+            if (j < v_group) *reinterpret_cast<uint4*>(dst + j) = *reinterpret_cast<const uint4*>(vals + j);
     }
 }
 
@@ -139,6 +170,8 @@ SIA_EXPORT int sia_rope_kv_write(void* qkv, int row_stride, const float* cos_tab
     if (rotary_dim > 0 && (!cos_table || !sin_table)) return SIA_BAD_ARGUMENT;
     dim3 grid(n_tokens);
     const bool vec = head_dim % 8 == 0 && rotary_dim % 16 == 0 && row_stride % 8 == 0;
+    // tokens whose values one workgroup writes together (0: every token its own); needs runs aligned to 16 bytes
+    const int v_group = (n_kv > 0 && n_tokens > 1 && page_size % 16 == 0) ? 16 : (n_kv > 0 && n_tokens > 1 && page_size % 8 == 0) ? 8 : 0;
     const int items = vec ? (n_heads + n_kv) * (rotary_dim / 16) + n_kv * ((head_dim - rotary_dim) / 8 + head_dim / 8) : 0;
     dim3 block(vec ? min(1024, max(SIA_WAVE, (items + SIA_WAVE - 1) / SIA_WAVE * SIA_WAVE)) : 256);
 #define LAUNCH(T)                                                                                             \
@@ -146,7 +179,8 @@ SIA_EXPORT int sia_rope_kv_write(void* qkv, int row_stride, const float* cos_tab
         if (vec)                                                                                              \
             hipLaunchKernelGGL(rope_kv_write_vec_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride,      \
                                cos_table, sin_table, positions, seq_of_token, block_table, table_width,       \
-                               (T*)k_pages, (T*)v_pages, n_heads, n_kv, head_dim, rotary_dim, page_size);     \
+                               (T*)k_pages, (T*)v_pages, n_heads, n_kv, head_dim, rotary_dim, page_size,      \
+                               v_group);                                                                      \
         else                                                                                                  \
             hipLaunchKernelGGL(rope_kv_write_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride,          \
                                cos_table, sin_table, positions, seq_of_token, block_table, table_width,       \
