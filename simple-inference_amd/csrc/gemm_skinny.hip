@@ -21,8 +21,8 @@
 // traffic) and rows m >= M of X the last live one; what the MFMAs make of them is never stored.
 //
 // The result element (m, n) is summed over k in an order that depends on K only, not on M, the other rows,
-// the number of waves, the row blocks of a workgroup or the depth of its pipeline: whichever shape a launch
-// takes, a row's result is the same bit for bit.
+// the number of waves, the row blocks of a workgroup or their height: whichever shape a launch takes, a row's
+// result is the same bit for bit.
 #include "common.h"
 
 #include <initializer_list>
@@ -57,7 +57,7 @@ struct ResidualOut {
     float* residual;      // [M][N], updated in place
     const float* gain;    // [N], the norm's weight
     bf16_t* scaled;       // [M][N] = residual * gain, not yet divided by the row's root mean square
-    float* partials;      // [N / 16][16]: sum over 16 columns of residual^2, by row
+    float* partials;      // [column blocks][16]: sum over a block's columns of residual^2, by row
 };
 
 // X is such a `scaled` matrix: row m of the result is to be multiplied by rsqrt(sum_p partials[p][m] / K + eps).
@@ -83,8 +83,8 @@ struct Epilogue {
 //                rounded product, so the two paths differ by a rounding); q goes to Y, k and v into the pages.
 //   EPI_RESIDUAL: the result, rounded as EPI_STORE rounds it, is added to the float residual; Y is not written.
 //                RMSNorm(x) W^T = rsqrt(mean x^2 + eps) * ((x * gain) W^T): the kernel leaves x * gain and the sums
-//                of squares of its own 16-column blocks, and the product after it (SCALED) adds those up, in an
-//                order that depends on N only, and scales its rows: no kernel of its own for the norm.
+//                of squares of its own column blocks, and the product after it (SCALED) adds those up, in an
+//                order that depends on their number only, and scales its rows: no kernel of its own for the norm.
 // Output columns come in *units*: a column of Y (EPI_STORE, EPI_RESIDUAL, EPI_SWIGLU, where unit u needs row u of
 // the gate half and row u of the up half of W), or a pair of columns that the rotation mixes (EPI_ROPE: unit u is
 // column u % (head_dim / 2) of head u / (head_dim / 2) together with the column head_dim / 2 further).  A workgroup
