@@ -490,13 +490,15 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
 // ---------------------------------------------------------------------------------------------------
 // prefill: runs of several tokens (works for single tokens too, without splitting the keys)
 // ---------------------------------------------------------------------------------------------------
-// Three shapes of workgroup.  Wide: 128 tokens, 4 waves of 32 tokens each, one tile of keys a step (fewest
+// Four shapes of workgroup.  Wide: 128 tokens, 4 waves of 32 tokens each, one tile of keys a step (fewest
 // instructions and reads from LDS per MFMA: the fastest when there are workgroups enough to keep two on every
-// compute unit).  Eight waves of 16 tokens: two waves a SIMD from the start, so that one's softmax runs beside
-// the other's MFMAs.  Split: 64 tokens, 8 waves: waves 0-3 take 16 tokens each and the even tiles of keys,
-// waves 4-7 the same tokens and the odd tiles, two tiles a step, and the two halves are merged through LDS at
-// the end: half as many steps for the last tokens of a prompt, whose many keys set the time of a short prompt
-// or portion.  Head sizes above 128 take 4 waves of 16 tokens.
+// compute unit).  Split: 64 tokens, 8 waves: waves 0-3 take 16 tokens each and the even tiles of keys, waves 4-7
+// the same tokens and the odd tiles, two tiles a step, and the two halves are merged through LDS at the end: half
+// as many steps for the last tokens of a prompt, whose many keys set the time of a short prompt or portion.
+// Paired: the same with 32 tokens a wave (128 tokens a workgroup), between the two: half the steps of the wide
+// shape, half the reads from LDS per MFMA of the split one (6 to 8 % faster than 8 waves of 16 tokens that each
+// take every tile, from 1,280 to 2,560 tokens at 24 heads).  Long: 256 tokens, 8 waves of 32.  Head sizes above
+// 128 take 4 waves of 16 tokens.
 constexpr int PF_ROWS = HD <= 128 ? 128 : 64;  // tokens per wide workgroup
 constexpr int PF_ROWS_SPLIT = 64;              // tokens per split workgroup
 constexpr int PF_ROWS_LONG = 256;              // tokens per workgroup of 8 waves of 32 tokens
@@ -937,14 +939,14 @@ SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_p
     } else {
         // Which shape is the fastest follows the number of workgroups per compute unit (measured at 24 heads of 128
         // on 256 compute units): the split shape while all its workgroups are on the chip at once (under 7/8 of a
-        // wide workgroup per compute unit: prompts or portions up to about 1,024 tokens), the 8-wave shape of 128
-        // tokens (two tiles of keys a step) up to 15/8 (about 2,048 tokens), the wide shape (one tile a step)
-        // beyond, and from 75/8 on (about 12,000 tokens) 8 waves of 32 tokens (256 tokens a workgroup, two tiles a
-        // step: a tile staged in LDS then serves twice as many tokens).
+        // wide workgroup per compute unit: prompts or portions up to about 1,024 tokens), the paired shape of 128
+        // tokens (two tiles of keys a step, one for each set of waves) up to 15/8 (about 2,500 tokens), the wide
+        // shape (one tile a step) beyond, and from 75/8 on (about 12,000 tokens) 8 waves of 32 tokens (256 tokens a
+        // workgroup, two tiles a step: a tile staged in LDS then serves twice as many tokens).
         const long long wide_groups = (long long)n_tiles * n_heads, cus = compute_units();
         if (PF_USE_LDS && n_tiles_split > 0 && wide_groups * 8 <= cus * 7)
             return launch_prefill<1, 2 * PF_ROWS_SPLIT / 16, 2>(n_tiles_split, ARGS);
-        if (wide_groups * 8 <= cus * 15) return launch_prefill<1, PF_ROWS / 16, 1, PF_USE_LDS ? 2 : 1>(n_tiles, ARGS);
+        if (PF_USE_LDS && wide_groups * 8 <= cus * 15) return launch_prefill<2, 2 * PF_ROWS / 32, 2, 2>(n_tiles, ARGS);
         if (PF_USE_LDS && n_tiles_long > 0 && wide_groups * 8 >= cus * 75)
             return launch_prefill<2, PF_ROWS_LONG / 32, 1, 2>(n_tiles_long, ARGS);
         return launch_prefill<2, PF_ROWS / 32, 1>(n_tiles, ARGS);
