@@ -497,7 +497,7 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
 // as many steps for the last tokens of a prompt, whose many keys set the time of a short prompt or portion.
 // Paired: the same with 32 tokens a wave (128 tokens a workgroup), between the two: half the steps of the wide
 // shape, half the reads from LDS per MFMA of the split one (6 to 8 % faster than 8 waves of 16 tokens that each
-// take every tile, from 1,280 to 2,560 tokens at 24 heads).  Long: 256 tokens, 8 waves of 32.  Head sizes above
+// take every tile, from 1,280 to 2,560 tokens at 24 heads; 10 to 17 % faster than the split shape from 1,024).  Long: 256 tokens, 8 waves of 32.  Head sizes above
 // 128 take 4 waves of 16 tokens.
 constexpr int PF_ROWS = HD <= 128 ? 128 : 64;  // tokens per wide workgroup
 constexpr int PF_ROWS_SPLIT = 64;              // tokens per split workgroup
@@ -938,13 +938,13 @@ SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_p
         return launch_prefill<1, PF_ROWS / 16, 1>(n_tiles, ARGS);
     } else {
         // Which shape is the fastest follows the number of workgroups per compute unit (measured at 24 heads of 128
-        // on 256 compute units): the split shape while all its workgroups are on the chip at once (under 7/8 of a
-        // wide workgroup per compute unit: prompts or portions up to about 1,024 tokens), the paired shape of 128
+        // on 256 compute units): the split shape while all its workgroups are on the chip at once (under 5/8 of a
+        // wide workgroup per compute unit: prompts or portions up to about 800 tokens), the paired shape of 128
         // tokens (two tiles of keys a step, one for each set of waves) up to 15/8 (about 2,500 tokens), the wide
         // shape (one tile a step) beyond, and from 75/8 on (about 12,000 tokens) 8 waves of 32 tokens (256 tokens a
         // workgroup, two tiles a step: a tile staged in LDS then serves twice as many tokens).
         const long long wide_groups = (long long)n_tiles * n_heads, cus = compute_units();
-        if (PF_USE_LDS && n_tiles_split > 0 && wide_groups * 8 <= cus * 7)
+        if (PF_USE_LDS && n_tiles_split > 0 && wide_groups * 8 <= cus * 5)
             return launch_prefill<1, 2 * PF_ROWS_SPLIT / 16, 2>(n_tiles_split, ARGS);
         if (PF_USE_LDS && wide_groups * 8 <= cus * 15) return launch_prefill<2, 2 * PF_ROWS / 32, 2, 2>(n_tiles, ARGS);
         if (PF_USE_LDS && n_tiles_long > 0 && wide_groups * 8 >= cus * 75)
