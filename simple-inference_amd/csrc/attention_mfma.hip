@@ -266,35 +266,45 @@ __device__ __forceinline__ void compute_stage(const Stage& st, const bf16x8 (&q)
             acc[n][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.v[db], p[n], acc[n][db], 0, 0, 0);
 }
 
+// Called before a tile is computed; the default does nothing.
+struct NoHook {
+    __device__ __forceinline__ void operator()(int) const {}
+};
+
 // The tiles w_first, w_first + TILE, ..., w_last, whose block-table entries the window holds; two register
-// stages in turn: the loads of tile t+1 are issued before the arithmetic of tile t.
-template <int NQ>
+// stages in turn: the loads of tile t+1 are issued before the arithmetic of tile t.  `before(kb)` runs before the
+// arithmetic of the tile at kb (it may hand the state on and start it afresh).
+template <int NQ, typename Hook>
 __device__ __forceinline__ void attend_tiles(const PageWindow& pages, int w_first, int w_last,
                                              const bf16x8 (&q)[NQ][KSTEPS], const bf16_t* __restrict__ kp,
                                              const bf16_t* __restrict__ vp, int ps_log2, int n_kv, int hk,
                                              int range_lo, int range_hi, const int (&lo)[NQ], const int (&hi)[NQ],
-                                             float scale, Softmax<NQ>& sm, floatx4 (&acc)[NQ][DBLOCKS]) {
+                                             float scale, Softmax<NQ>& sm, floatx4 (&acc)[NQ][DBLOCKS], Hook& before) {
     Stage a, b;
     load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, w_first, range_lo, range_hi);
     for (int kb = w_first; kb <= w_last; kb += 2 * TILE) {
         const int kb1 = min(kb + TILE, w_last);  // past the end: the last tile again, never computed
         load_stage(b, kp, vp, pages, ps_log2, n_kv, hk, kb1, range_lo, range_hi);
+        before(kb);
         compute_stage<NQ>(a, q, kb, lo, hi, scale, sm, acc);
         const int kb2 = min(kb + 2 * TILE, w_last);
         load_stage(a, kp, vp, pages, ps_log2, n_kv, hk, kb2, range_lo, range_hi);
-        if (kb + TILE <= w_last) compute_stage<NQ>(b, q, kb + TILE, lo, hi, scale, sm, acc);
+        if (kb + TILE <= w_last) {
+            before(kb + TILE);
+            compute_stage<NQ>(b, q, kb + TILE, lo, hi, scale, sm, acc);
+        }
     }
 }
 
 // All tiles that meet [range_lo, range_hi] (range_lo <= range_hi).  The block-table window (64 entries,
 // starting at the page of the first tile it serves) is loaded outside the pipelined loop, once per 64
 // pages: a load inside it would make every iteration wait for all outstanding loads.
-template <int NQ>
+template <int NQ, typename Hook>
 __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], const bf16_t* __restrict__ kp,
                                              const bf16_t* __restrict__ vp, const int* __restrict__ table,
                                              int table_width, int ps_log2, int n_kv, int hk, int range_lo,
                                              int range_hi, const int (&lo)[NQ], const int (&hi)[NQ], float scale,
-                                             Softmax<NQ>& sm, floatx4 (&acc)[NQ][DBLOCKS]) {
+                                             Softmax<NQ>& sm, floatx4 (&acc)[NQ][DBLOCKS], Hook& before) {
     const int lane = threadIdx.x & 63;
     const int kb_first = (range_lo / TILE) * TILE, kb_last = (range_hi / TILE) * TILE;
     for (int w_first = kb_first; w_first <= kb_last;) {
@@ -303,9 +313,20 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], cons
         PageWindow pages;
         pages_load(pages, table, table_width, first_page, lane);
         attend_tiles<NQ>(pages, w_first, min(kb_last, w_end - TILE), q, kp, vp, ps_log2, n_kv, hk, range_lo, range_hi,
-                         lo, hi, scale, sm, acc);
+                         lo, hi, scale, sm, acc, before);
         w_first = w_end;
     }
+}
+
+template <int NQ>
+__device__ __forceinline__ void attend_range(const bf16x8 (&q)[NQ][KSTEPS], const bf16_t* __restrict__ kp,
+                                             const bf16_t* __restrict__ vp, const int* __restrict__ table,
+                                             int table_width, int ps_log2, int n_kv, int hk, int range_lo,
+                                             int range_hi, const int (&lo)[NQ], const int (&hi)[NQ], float scale,
+                                             Softmax<NQ>& sm, floatx4 (&acc)[NQ][DBLOCKS]) {
+    NoHook none;
+    attend_range<NQ>(q, kp, vp, table, table_width, ps_log2, n_kv, hk, range_lo, range_hi, lo, hi, scale, sm, acc,
+                     none);
 }
 
 // q operand of column r: 8 dims d0 .. d0+7 of that column's query row (zeros if the column is unused).
@@ -353,22 +374,60 @@ __device__ __forceinline__ float merge_splits(int n_splits, float mx, At at) {
     return o * (1.f / denom);
 }
 
-// Grid (kv heads, sequences, splits), or with `fold` (kv heads, sequences, 1): a workgroup then takes the splits of
-// its (sequence, kv head) one after the other, keeps their results in LDS and merges them itself, the way the
-// combine kernel does, bit for bit.  For steps of so many sequences that the splits are not needed to fill the
-// device: no partial results in memory and no second kernel.
+// What the DEC_WAVES waves of one split left in LDS (rows[w * group + c] = acc[HD], m, l), merged for element d of
+// query head c of the group: the split's (acc, m, l).  The same arithmetic wherever it is called from.
+__device__ __forceinline__ void merge_waves(const float* rows, int group, int c, int d, float& o, float& mx,
+                                            float& lsum) {
+    constexpr int ROW = HD + 2;
+    mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, rows[(size_t)(w * group + c) * ROW + HD]);
+    const float mx_use = (mx == -INFINITY) ? 0.f : mx;  // no wave had a key: all weights 0, the split counts for nothing
+    o = 0.f;
+    lsum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const float* row = rows + (size_t)(w * group + c) * ROW;
+        const float wgt = fast_exp2(row[HD] - mx_use);  // a wave without keys has m = -inf: weight 0
+        o += wgt * row[d];
+        lsum += wgt * row[HD + 1];
+    }
+}
+
+// One wave's state, finished, into its row of LDS (lanes whose column is no query head of the group write nothing).
+__device__ __forceinline__ void leave_state(float* mine, Softmax<1>& sm, const floatx4 (&acc)[1][DBLOCKS], int g,
+                                            bool writes) {
+    sm.finish_sums();
+    if (!writes) return;
+    if (g == 0) {
+        mine[HD] = sm.m[0];
+        mine[HD + 1] = sm.l[0];
+    }
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mine[db * 16 + g * 4 + i] = acc[0][db][i];
+}
+
+// Grid (kv heads, sequences, splits), or with `fold` (kv heads, sequences, 1).  A sequence's visible key tiles are
+// dealt evenly, in order, to n_splits * DEC_WAVES runs (every run contiguous, runs differ by one tile at most);
+// the four runs of a split are merged, then the splits.  Without `fold` a workgroup is one split, a wave one run,
+// and the combine kernel merges the splits.  With `fold` one workgroup does it all: each of its waves walks
+// n_splits runs that follow one another as one stream of tiles (its loads never stop at a run's end), leaves each
+// run's state in LDS as it passes the run's end, and the workgroup merges runs and splits itself, with the same
+// arithmetic, bit for bit.  For steps of so many sequences that the splits are not needed to fill the device: no
+// partial results in memory and no second kernel.
 __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
     bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window, int max_splits, int fold) {
-    extern __shared__ float lds[];  // [DEC_WAVES][group][HD + 2], with fold then [max_splits][group][HD + 2]
+    static_assert(DEC_WAVES == 4, "merge_waves merges four runs");
+    extern __shared__ float lds[];  // [runs of the workgroup][group][HD + 2]
     // splits are the slowest index of the grid: the workgroups that leave at once (splits a sequence does not
     // have) then come last, not interleaved with the others, which the chip deals out to its dies in turn
     const int hk = blockIdx.x, seq = blockIdx.y;
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
-    // The tiles that hold visible keys are dealt evenly, in order, to the n_splits * DEC_WAVES waves that
-    // work for this (sequence, kv head): every wave gets a contiguous run, runs differ by one tile at most.
     const int pos = kv_len[seq] - 1;
     const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
     const int t_first = lo_all / TILE, n_tiles = pos / TILE - t_first + 1;
@@ -379,90 +438,76 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const int* table = block_table + (size_t)seq * table_width;
     bf16x8 qf[1][KSTEPS];
     load_q(qf[0], r < group ? q + (size_t)seq * q_row_stride + (hk * group + r) * HD : nullptr, g);
-    const int n_waves = n_splits * DEC_WAVES;
+    const int n_runs = n_splits * DEC_WAVES;
     constexpr int ROW = HD + 2;
-    float* const kept = lds + (size_t)DEC_WAVES * group * ROW;  // with fold: the splits' results
+    auto run_begin = [&](int run) { return t_first + (int)(((long long)run * n_tiles) / n_runs); };  // its first tile
 
-    const int split_first = fold ? 0 : blockIdx.z, split_end = fold ? n_splits : blockIdx.z + 1;
-    for (int split = split_first; split < split_end; ++split) {
-        const int wi = split * DEC_WAVES + wave;
-        const int my_first = t_first + (int)(((long long)wi * n_tiles) / n_waves);
-        const int my_end = t_first + (int)(((long long)(wi + 1) * n_tiles) / n_waves);
-
-        Softmax<1> sm;
-        sm.start();
-        floatx4 acc[1][DBLOCKS];
+    // this wave's runs: one (of this workgroup's split), or with fold n_splits in a row
+    const int mine_n = fold ? n_splits : 1;
+    const int run0 = fold ? wave * n_splits : blockIdx.z * DEC_WAVES + wave;
+    const int first = run_begin(run0), end = run_begin(run0 + mine_n);
+    Softmax<1> sm;
+    sm.start();
+    floatx4 acc[1][DBLOCKS];
 #pragma unroll
-        for (int db = 0; db < DBLOCKS; ++db) acc[0][db] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-        if (my_first < my_end) {  // wave-uniform
-            const int w_lo = max(lo_all, my_first * TILE), w_hi = min(pos, my_end * TILE - 1);
-            const int lo[1] = {r < group ? w_lo : 1}, hi[1] = {r < group ? w_hi : 0};
-            attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, sm, acc);
+    for (int db = 0; db < DBLOCKS; ++db) acc[0][db] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // the row of LDS of run `run0 + j`: with fold rows are in order of runs, else the wave's own
+    auto row_of = [&](int j) { return lds + (size_t)((fold ? run0 + j : wave) * group + min(r, group - 1)) * ROW; };
+    struct AtRunEnds {  // before the tile at kb: every run that ends at or before it hands its state on
+        int done, run_end;
+        const int mine_n, run0, r, g, group;
+        Softmax<1>& sm;
+        floatx4 (&acc)[1][DBLOCKS];
+        decltype(run_begin)& begin;
+        decltype(row_of)& row;
+        __device__ __forceinline__ void pass() {
+            float* mine = row(done);
+            Softmax<1> left = sm;
+            leave_state(mine, left, acc, g, r < group);
+            sm.start();
+#pragma unroll
+            for (int db = 0; db < DBLOCKS; ++db) acc[0][db] = floatx4{0.f, 0.f, 0.f, 0.f};
+            ++done;
+            run_end = begin(run0 + done + 1);
         }
-        sm.finish_sums();
-
-        if (split != split_first) __syncthreads();  // the split before has been read out of the waves' rows
-        if (r < group) {
-            float* mine = lds + (size_t)(wave * group + r) * ROW;
-            if (g == 0) {
-                mine[HD] = sm.m[0];
-                mine[HD + 1] = sm.l[0];
-            }
-#pragma unroll
-            for (int db = 0; db < DBLOCKS; ++db)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) mine[db * 16 + g * 4 + i] = acc[0][db][i];
+        __device__ __forceinline__ void operator()(int kb) {
+            while (done < mine_n - 1 && kb / TILE >= run_end) pass();  // wave-uniform
         }
-        __syncthreads();
-        for (int idx = threadIdx.x; idx < group * HD; idx += DEC_WAVES * SIA_WAVE) {
-            const int c = idx / HD, d = idx % HD;
-            float mx = -INFINITY;
-#pragma unroll
-            for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, lds[(size_t)(w * group + c) * ROW + HD]);
-            const float mx_use = (mx == -INFINITY) ? 0.f : mx;  // no wave had a key: all weights 0, the split counts for nothing
-            float o = 0.f, lsum = 0.f;
-#pragma unroll
-            for (int w = 0; w < DEC_WAVES; ++w) {
-                const float* row = lds + (size_t)(w * group + c) * ROW;
-                const float wgt = fast_exp2(row[HD] - mx_use);  // a wave without keys has m = -inf: weight 0
-                o += wgt * row[d];
-                lsum += wgt * row[HD + 1];
-            }
+    } at_run_ends{0, run_begin(run0 + 1), mine_n, run0, r, g, group, sm, acc, run_begin, row_of};
+
+    if (first < end) {  // wave-uniform
+        const int w_lo = max(lo_all, first * TILE), w_hi = min(pos, end * TILE - 1);
+        const int lo[1] = {r < group ? w_lo : 1}, hi[1] = {r < group ? w_hi : 0};
+        attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, sm, acc,
+                        at_run_ends);
+    }
+    while (at_run_ends.done < mine_n - 1) at_run_ends.pass();  // runs without tiles of their own
+    leave_state(row_of(mine_n - 1), sm, acc, g, r < group);
+    __syncthreads();
+
+    for (int idx = threadIdx.x; idx < group * HD; idx += DEC_WAVES * SIA_WAVE) {
+        const int c = idx / HD, d = idx % HD;
+        bf16_t* dst = out + ((size_t)cu_q[seq] * n_heads + hk * group + c) * HD + d;
+        if (!fold || n_splits == 1) {
+            float o, mx, lsum;
+            merge_waves(lds, group, c, d, o, mx, lsum);
             if (n_splits == 1) {  // nothing to combine with: this is the result
-                out[((size_t)cu_q[seq] * n_heads + hk * group + c) * HD + d] = float_to_bf16(o * (1.f / lsum));
+                *dst = float_to_bf16(o * (1.f / lsum));
                 continue;
             }
-            if (fold) {
-                float* row = kept + (size_t)(split * group + c) * ROW;
-                row[d] = o;
-                if (d == 0) {
-                    row[HD] = mx;
-                    row[HD + 1] = lsum;
-                }
-                continue;
-            }
-            const size_t slot = ((size_t)seq * n_heads + hk * group + c) * max_splits + split;
+            const size_t slot = ((size_t)seq * n_heads + hk * group + c) * max_splits + blockIdx.z;
             ws_acc[slot * HD + d] = o;
             if (d == 0) {
                 ws_ml[slot * 2] = mx;
                 ws_ml[slot * 2 + 1] = lsum;
             }
+            continue;
         }
-    }
-    if (!fold || n_splits == 1) return;
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < group * HD; idx += DEC_WAVES * SIA_WAVE) {
-        const int c = idx / HD, d = idx % HD;
-        float mx = -INFINITY;
-        for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, kept[(size_t)(s * group + c) * ROW + HD]);
-        const float o = merge_splits(n_splits, mx, [&](int s, float& acc, float& m, float& l) {
-            const float* row = kept + (size_t)(s * group + c) * ROW;
-            acc = row[d];
-            m = row[HD];
-            l = row[HD + 1];
-        });
-        out[((size_t)cu_q[seq] * n_heads + hk * group + c) * HD + d] = float_to_bf16(o);
+        float mx_all = -INFINITY;
+        for (int run = 0; run < n_runs; ++run) mx_all = fmaxf(mx_all, lds[(size_t)(run * group + c) * ROW + HD]);
+        *dst = float_to_bf16(merge_splits(n_splits, mx_all, [&](int sp, float& a, float& m, float& l) {
+            merge_waves(lds + (size_t)sp * DEC_WAVES * group * ROW, group, c, d, a, m, l);
+        }));
     }
 }
 
@@ -867,11 +912,11 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
     size_t lds_bytes = DEC_WAVES * row_bytes;
     if (lds_bytes > 64 * 1024) return SIA_BAD_ARGUMENT;
     // With two workgroups or more for every compute unit without them, the splits of a (sequence, kv head) are
-    // taken by one workgroup in turn (if their results fit into its LDS): the same numbers, one kernel.
+    // taken by one workgroup (if the states of all their runs fit into its LDS): the same numbers, one kernel.
     const bool fold = n_splits > 1 && (long long)n_kv * n_seqs >= 2ll * compute_units() &&
-                      lds_bytes + n_splits * row_bytes <= 64 * 1024;
+                      lds_bytes * n_splits <= 64 * 1024;
     if (fold) {
-        lds_bytes += n_splits * row_bytes;
+        lds_bytes *= n_splits;  // a row for every run
         if (lds_bytes > 48 * 1024) {  // beyond the default limit of dynamic LDS
             static bool allowed[64];
             int device = 0;
