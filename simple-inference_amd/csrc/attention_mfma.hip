@@ -911,9 +911,9 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
     const size_t row_bytes = (size_t)(n_heads / n_kv) * (HD + 2) * sizeof(float);
     size_t lds_bytes = DEC_WAVES * row_bytes;
     if (lds_bytes > 64 * 1024) return SIA_BAD_ARGUMENT;
-    // With two workgroups or more for every compute unit without them, the splits of a (sequence, kv head) are
+    // With a workgroup or more for every compute unit without them, the splits of a (sequence, kv head) are
     // taken by one workgroup (if the states of all their runs fit into its LDS): the same numbers, one kernel.
-    const bool fold = n_splits > 1 && (long long)n_kv * n_seqs >= 2ll * compute_units() &&
+    const bool fold = n_splits > 1 && (long long)n_kv * n_seqs >= compute_units() &&
                       lds_bytes * n_splits <= 64 * 1024;
     if (fold) {
         lds_bytes *= n_splits;  // a row for every run
