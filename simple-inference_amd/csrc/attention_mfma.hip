@@ -632,14 +632,31 @@ __device__ __forceinline__ void tile_store(const TileRegs<TEAM>& t, bf16_t* __re
     }
 }
 
-// Scores, online softmax and value product of one tile held in an LDS stage; every operand is read
-// right before the MFMAs that use it.
-template <int NQ>
+// Scores, online softmax and value product of one tile held in an LDS stage.  With EARLY all key operands of the
+// tile are read before the first score MFMA and all value operands before the softmax, so that a read's latency
+// passes behind the arithmetic in front of it instead of in front of the two MFMAs that use it (4 % at 2,048 tokens;
+// these shapes hold one workgroup a compute unit whatever they do, so the registers are there); without it every
+// operand is read right before its MFMAs, which the 256-token shape, that has most arithmetic per read, likes
+// better by 3 %.
+template <int NQ, bool EARLY>
 __device__ __forceinline__ void compute_from_lds(const bf16_t* __restrict__ k_lds, const bf16_t* __restrict__ v_lds,
                                                  const bf16x8 (&q)[NQ][KSTEPS], int kb, const int (&lo)[NQ],
                                                  const int (&hi)[NQ], float scale, Softmax<NQ>& sm,
                                                  floatx4 (&acc)[NQ][DBLOCKS]) {
     const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    auto key_operand = [&](int h, int ks) {
+        const int d0 = ks * 32 + g * 8;
+        if (HD % 32 == 0 || ks < KSTEPS - 1) return load8(k_lds + (h * 16 + r) * K_STRIDE + d0);
+        return d0 < HD ? load8(k_lds + (h * 16 + r) * K_STRIDE + d0) : zero8();
+    };
+    auto value_operand = [&](int db) { return load8(v_lds + (db * 16 + r) * V_STRIDE + g * 8); };
+    bf16x8 ka[2][KSTEPS], va[DBLOCKS];
+    if (EARLY) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) ka[h][ks] = key_operand(h, ks);
+    }
     floatx4 s[NQ][2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -647,21 +664,20 @@ __device__ __forceinline__ void compute_from_lds(const bf16_t* __restrict__ k_ld
         for (int n = 0; n < NQ; ++n) s[n][h] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
-            const int d0 = ks * 32 + g * 8;
-            bf16x8 a;
-            if (HD % 32 == 0 || ks < KSTEPS - 1)
-                a = load8(k_lds + (h * 16 + r) * K_STRIDE + d0);
-            else
-                a = d0 < HD ? load8(k_lds + (h * 16 + r) * K_STRIDE + d0) : zero8();
+            const bf16x8 a = EARLY ? ka[h][ks] : key_operand(h, ks);
 #pragma unroll
             for (int n = 0; n < NQ; ++n) s[n][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[n][ks], s[n][h], 0, 0, 0);
         }
+    }
+    if (EARLY) {
+#pragma unroll
+        for (int db = 0; db < DBLOCKS; ++db) va[db] = value_operand(db);
     }
     bf16x8 p[NQ];
     softmax_update<NQ>(s, kb, lo, hi, scale, sm, acc, p);
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) {
-        const bf16x8 a = load8(v_lds + (db * 16 + r) * V_STRIDE + g * 8);
+        const bf16x8 a = EARLY ? va[db] : value_operand(db);
 #pragma unroll
         for (int n = 0; n < NQ; ++n) acc[n][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p[n], acc[n][db], 0, 0, 0);
     }
@@ -742,6 +758,7 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
         const int kb_first = (blk_lo / TILE) * TILE, kb_last = (blk_hi / TILE) * TILE;
         constexpr int STEP_KEYS = KTILES * TILE;
         constexpr int AHEAD = PF_NQ == 1 ? 4 : 2;
+        constexpr bool EARLY = KSPLIT == 2 || KTILES == 1;  // all shapes but the one of 256 tokens
         static_assert(AHEAD % 2 == 0, "the LDS stage of a step is its parity within a group of AHEAD");
         FetchPlan<TEAM> plan;
         plan.make(ps_log2, hk);
@@ -776,8 +793,8 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
             if (p % KSPLIT != part) continue; /* each set of waves its tiles of the step */                     \
             const int my_kb = (KB) + p * TILE;                                                                  \
             if (wave_live && my_kb <= w_last && my_kb <= wave_hi && my_kb + TILE - 1 >= wave_lo)                \
-                compute_from_lds<PF_NQ>(PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), qf, my_kb, lo, hi, scale, sm,   \
-                                        acc);                                                                   \
+                compute_from_lds<PF_NQ, EARLY>(PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), qf, my_kb, lo, hi, scale, \
+                                               sm, acc);                                                        \
         }                                                                                                       \
         PF_STORE(NEXT, (KB) + STEP_KEYS, (STAGE) ^ 1);                                                          \
         __syncthreads();                                                                                        \
