@@ -344,6 +344,7 @@ __device__ __forceinline__ void load_q(bf16x8 (&q)[KSTEPS], const bf16_t* row, i
 constexpr int DEC_WAVES = 4;
 constexpr int DEC_TILES_PER_SPLIT = 16;  // a split is worth taking from this many tiles (512 keys) on
 constexpr int DEC_MAX_SPLITS = 32;
+constexpr int DEC_FOLD_LDS = 128 * 1024;  // most LDS a workgroup that does all splits may take for their states
 
 // Workgroups that share one (sequence, kv head) with n_tiles visible key tiles: the largest power of two that
 // leaves every workgroup DEC_TILES_PER_SPLIT tiles, at most DEC_MAX_SPLITS.  A function of the sequence's own
@@ -931,7 +932,7 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
     // With a workgroup or more for every compute unit without them, the splits of a (sequence, kv head) are
     // taken by one workgroup (if the states of all their runs fit into its LDS): the same numbers, one kernel.
     const bool fold = n_splits > 1 && (long long)n_kv * n_seqs >= compute_units() &&
-                      lds_bytes * n_splits <= 64 * 1024;
+                      lds_bytes * n_splits <= DEC_FOLD_LDS;
     if (fold) {
         lds_bytes *= n_splits;  // a row for every run
         if (lds_bytes > 48 * 1024) {  // beyond the default limit of dynamic LDS
@@ -940,7 +941,7 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
             if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return SIA_BAD_ARGUMENT;
             if (!allowed[device]) {
                 const hipError_t e = hipFuncSetAttribute((const void*)attn_decode_kernel,
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, DEC_FOLD_LDS);
                 if (e != hipSuccess) return (int)e;
                 allowed[device] = true;
             }
