@@ -375,23 +375,24 @@ __device__ __forceinline__ float merge_splits(int n_splits, float mx, At at) {
     return o * (1.f / denom);
 }
 
-// What the DEC_WAVES waves of one split left in LDS (rows[w * group + c] = acc[HD], m, l), merged for element d of
-// query head c of the group: the split's (acc, m, l).  The same arithmetic wherever it is called from.
-__device__ __forceinline__ void merge_waves(const float* rows, int group, int c, int d, float& o, float& mx,
-                                            float& lsum) {
-    constexpr int ROW = HD + 2;
+// The states of the four runs of one split, merged for one element of one query head: the split's (acc, m, l).
+// `row(w)` is run w's state of that head: acc[HD], m, l.  The same arithmetic wherever it is called from.
+template <typename Row>
+__device__ __forceinline__ void merge_waves(Row row, int d, float& o, float& mx, float& lsum) {
+    const float* rows[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) rows[w] = row(w);
     mx = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, rows[(size_t)(w * group + c) * ROW + HD]);
-    const float mx_use = (mx == -INFINITY) ? 0.f : mx;  // no wave had a key: all weights 0, the split counts for nothing
+    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, rows[w][HD]);
+    const float mx_use = (mx == -INFINITY) ? 0.f : mx;  // no run had a key: all weights 0, the split counts for nothing
     o = 0.f;
     lsum = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-        const float* row = rows + (size_t)(w * group + c) * ROW;
-        const float wgt = fast_exp2(row[HD] - mx_use);  // a wave without keys has m = -inf: weight 0
-        o += wgt * row[d];
-        lsum += wgt * row[HD + 1];
+        const float wgt = fast_exp2(rows[w][HD] - mx_use);  // a run without keys has m = -inf: weight 0
+        o += wgt * rows[w][d];
+        lsum += wgt * rows[w][HD + 1];
     }
 }
 
@@ -410,19 +411,27 @@ __device__ __forceinline__ void leave_state(float* mine, Softmax<1>& sm, const f
         for (int i = 0; i < 4; ++i) mine[db * 16 + g * 4 + i] = acc[0][db][i];
 }
 
-// Grid (kv heads, sequences, splits), or with `fold` (kv heads, sequences, 1).  A sequence's visible key tiles are
-// dealt evenly, in order, to n_splits * DEC_WAVES runs (every run contiguous, runs differ by one tile at most);
-// the four runs of a split are merged, then the splits.  Without `fold` a workgroup is one split, a wave one run,
-// and the combine kernel merges the splits.  With `fold` one workgroup does it all: each of its waves walks
-// n_splits runs that follow one another as one stream of tiles (its loads never stop at a run's end), leaves each
-// run's state in LDS as it passes the run's end, and the workgroup merges runs and splits itself, with the same
-// arithmetic, bit for bit.  For steps of so many sequences that the splits are not needed to fill the device: no
-// partial results in memory and no second kernel.
+// A sequence's visible key tiles are dealt evenly, in order, to n_splits * DEC_WAVES runs (every run contiguous,
+// runs differ by one tile at most); the four runs of a split are merged, then the splits, always with the same
+// arithmetic, so that how the runs are spread over workgroups changes no bit:
+//   DEC_PLAIN   grid (kv heads, sequences, splits), 4 waves: a workgroup is one split, a wave one run; the combine
+//               kernel merges the splits.
+//   DEC_FOLD    grid (kv heads, sequences, 1), 4 waves: one workgroup does it all.  Each of its waves walks n_splits
+//               runs that follow one another as one stream of tiles (its loads never stop at a run's end), leaves
+//               each run's state in LDS as it passes the run's end, and the workgroup merges runs and splits
+//               itself.  For steps of so many sequences that the splits are not needed to fill the device: no
+//               partial results in memory and no second kernel.
+//   DEC_SPREAD  grid (kv heads, sequences, runs), 1 wave: a workgroup is one run and leaves its state in the
+//               workspace; the combine kernel merges runs and splits.  For steps of so few sequences that their
+//               splits alone leave most compute units idle.
+enum DecodeMode { DEC_PLAIN = 0, DEC_FOLD = 1, DEC_SPREAD = 2 };
+
 __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
-    bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window, int max_splits, int fold) {
+    bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window, int max_splits, int mode) {
+    const bool fold = mode == DEC_FOLD, spread = mode == DEC_SPREAD;
     static_assert(DEC_WAVES == 4, "merge_waves merges four runs");
     extern __shared__ float lds[];  // [runs of the workgroup][group][HD + 2]
     // splits are the slowest index of the grid: the workgroups that leave at once (splits a sequence does not
@@ -433,7 +442,8 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
     const int t_first = lo_all / TILE, n_tiles = pos / TILE - t_first + 1;
     const int n_splits = min(decode_splits(n_tiles), max_splits);
-    if (!fold && (int)blockIdx.z >= n_splits) return;  // the whole workgroup: the grid is sized for the longest sequence there may be
+    // the whole workgroup leaves: the grid is sized for the longest sequence there may be
+    if (!fold && (int)blockIdx.z >= (spread ? n_splits * DEC_WAVES : n_splits)) return;
     scale *= LOG2E;  // exponentials are taken as powers of two
     const int group = n_heads / n_kv;
     const int* table = block_table + (size_t)seq * table_width;
@@ -445,7 +455,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
 
     // this wave's runs: one (of this workgroup's split), or with fold n_splits in a row
     const int mine_n = fold ? n_splits : 1;
-    const int run0 = fold ? wave * n_splits : blockIdx.z * DEC_WAVES + wave;
+    const int run0 = fold ? wave * n_splits : spread ? blockIdx.z : blockIdx.z * DEC_WAVES + wave;
     const int first = run_begin(run0), end = run_begin(run0 + mine_n);
     Softmax<1> sm;
     sm.start();
@@ -483,6 +493,11 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
                         at_run_ends);
     }
     while (at_run_ends.done < mine_n - 1) at_run_ends.pass();  // runs without tiles of their own
+    if (spread) {  // the run's state of every query head of the group: [sequence][head][run][HD + 2] in ws_acc
+        const size_t slot = ((size_t)seq * n_heads + hk * group + min(r, group - 1)) * (max_splits * DEC_WAVES) + run0;
+        leave_state(ws_acc + slot * ROW, sm, acc, g, r < group);
+        return;
+    }
     leave_state(row_of(mine_n - 1), sm, acc, g, r < group);
     __syncthreads();
 
@@ -491,7 +506,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
         bf16_t* dst = out + ((size_t)cu_q[seq] * n_heads + hk * group + c) * HD + d;
         if (!fold || n_splits == 1) {
             float o, mx, lsum;
-            merge_waves(lds, group, c, d, o, mx, lsum);
+            merge_waves([&](int w) { return lds + (size_t)(w * group + c) * ROW; }, d, o, mx, lsum);
             if (n_splits == 1) {  // nothing to combine with: this is the result
                 *dst = float_to_bf16(o * (1.f / lsum));
                 continue;
@@ -507,24 +522,38 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
         float mx_all = -INFINITY;
         for (int run = 0; run < n_runs; ++run) mx_all = fmaxf(mx_all, lds[(size_t)(run * group + c) * ROW + HD]);
         *dst = float_to_bf16(merge_splits(n_splits, mx_all, [&](int sp, float& a, float& m, float& l) {
-            merge_waves(lds + (size_t)sp * DEC_WAVES * group * ROW, group, c, d, a, m, l);
+            merge_waves([&](int w) { return lds + (size_t)((sp * DEC_WAVES + w) * group + c) * ROW; }, d, a, m, l);
         }));
     }
 }
 
-// Combines the splits of each (sequence, head) that workgroups of their own left in the workspaces.
+// Combines what workgroups of their own left in the workspaces for each (sequence, head): the splits' merged states
+// (ws_acc [..][split][HD], ws_ml [..][split][2]), or with `runs` the states of all runs (ws_acc [..][run][HD + 2]).
 __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
     const float* __restrict__ ws_acc, const float* __restrict__ ws_ml, const int* __restrict__ cu_q,
-    const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int max_splits, int window) {
+    const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int max_splits, int window, int runs) {
     const int head = blockIdx.x, seq = blockIdx.y, lane = threadIdx.x;
     const int pos = kv_len[seq] - 1;
     const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
     const int n_splits = min(decode_splits(pos / TILE - lo_all / TILE + 1), max_splits);
+    bf16_t* dst = out + ((size_t)cu_q[seq] * n_heads + head) * HD;
+    if (runs) {
+        constexpr int ROW = HD + 2;
+        const float* mine = ws_acc + ((size_t)seq * n_heads + head) * (max_splits * DEC_WAVES) * ROW;
+        float mx = -INFINITY;  // a lane a run: the loads go out together
+        for (int run = lane; run < n_splits * DEC_WAVES; run += SIA_WAVE) mx = fmaxf(mx, mine[(size_t)run * ROW + HD]);
+        mx = wave_max(mx);
+        for (int d = lane; d < HD; d += SIA_WAVE)
+            dst[d] = float_to_bf16(merge_splits(n_splits, mx, [&](int sp, float& acc, float& m, float& l) {
+                merge_waves([&](int w) { return mine + (size_t)(sp * DEC_WAVES + w) * ROW; }, d, acc, m, l);
+            }));
+        return;
+    }
     if (n_splits == 1) return;  // its one workgroup wrote the result itself
     const size_t base = ((size_t)seq * n_heads + head) * max_splits;
     float mx = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, ws_ml[(base + s) * 2]);
-    bf16_t* dst = out + ((size_t)cu_q[seq] * n_heads + head) * HD;
+    for (int s = lane; s < n_splits; s += SIA_WAVE) mx = fmaxf(mx, ws_ml[(base + s) * 2]);
+    mx = wave_max(mx);
     for (int d = lane; d < HD; d += SIA_WAVE)
         dst[d] = float_to_bf16(merge_splits(n_splits, mx, [&](int s, float& acc, float& m, float& l) {
             acc = ws_acc[(base + s) * HD + d];
@@ -911,10 +940,29 @@ SIA_EXPORT int sia_attn_decode_max_splits(int kv_bound, int window) {
     return decode_splits(tiles);
 }
 
+// How a decode step of n_seqs sequences, none with more splits than max_splits, spreads its runs over workgroups.
+static DecodeMode decode_mode(int n_seqs, int n_heads, int n_kv, int max_splits) {
+    const long long pairs = (long long)n_kv * n_seqs, cus = compute_units();
+    const size_t row_bytes = (size_t)(n_heads / n_kv) * (HD + 2) * sizeof(float);
+    if (max_splits > 1 && pairs >= cus && DEC_WAVES * row_bytes * max_splits <= (size_t)DEC_FOLD_LDS) return DEC_FOLD;
+    if (pairs * max_splits <= cus) return DEC_SPREAD;  // no more splits than compute units: a workgroup for every run
+    return DEC_PLAIN;
+}
+
+// Floats of ws_acc and of ws_ml that sia_attn_decode needs for such a step (0: none, the pointer may be null).
+SIA_EXPORT long long sia_attn_decode_workspace(int n_seqs, int n_heads, int n_kv, int max_splits, int which) {
+    if (n_seqs <= 0 || n_kv <= 0 || n_heads % n_kv || max_splits <= 0) return 0;
+    const long long states = (long long)n_seqs * n_heads;
+    switch (decode_mode(n_seqs, n_heads, n_kv, max_splits)) {
+    case DEC_FOLD: return 0;
+    case DEC_SPREAD: return which == 0 ? states * max_splits * DEC_WAVES * (HD + 2) : 0;
+    default: return max_splits > 1 ? states * max_splits * (which == 0 ? HD : 2) : 0;
+    }
+}
+
 // Sequences 0 .. n_seqs-1 of the step, each with exactly one new token, which is row s of q (cu_q[s] = s), and
-// none longer than kv_bound.  max_splits = sia_attn_decode_max_splits(kv_bound, window); ws_acc holds n_seqs *
-// n_heads * max_splits * head_dim floats, ws_ml n_seqs * n_heads * max_splits * 2 (neither is read before it is
-// written).
+// none longer than kv_bound.  max_splits = sia_attn_decode_max_splits(kv_bound, window); ws_acc and ws_ml hold
+// sia_attn_decode_workspace(.., 0) and (.., 1) floats (neither is read before it is written).
 SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                                const int* block_table, int table_width, const int* cu_q, const int* kv_len,
                                void* out, float* ws_acc, float* ws_ml, int n_seqs, int n_heads, int n_kv,
@@ -923,17 +971,16 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
     const int ps_log2 = log2_exact(page_size);
     const int n_splits = max_splits;
     if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || n_splits <= 0 ||
-        n_splits > DEC_MAX_SPLITS || n_kv > 65535 || n_seqs > 65535 || q_row_stride % 8 || table_width <= 0 ||
-        (n_splits > 1 && (!ws_acc || !ws_ml)))
+        n_splits > DEC_MAX_SPLITS || n_kv > 65535 || n_seqs > 65535 || q_row_stride % 8 || table_width <= 0)
+        return SIA_BAD_ARGUMENT;
+    const DecodeMode mode = decode_mode(n_seqs, n_heads, n_kv, n_splits);
+    if ((sia_attn_decode_workspace(n_seqs, n_heads, n_kv, n_splits, 0) && !ws_acc) ||
+        (sia_attn_decode_workspace(n_seqs, n_heads, n_kv, n_splits, 1) && !ws_ml))
         return SIA_BAD_ARGUMENT;
     const size_t row_bytes = (size_t)(n_heads / n_kv) * (HD + 2) * sizeof(float);
     size_t lds_bytes = DEC_WAVES * row_bytes;
     if (lds_bytes > 64 * 1024) return SIA_BAD_ARGUMENT;
-    // With a workgroup or more for every compute unit without them, the splits of a (sequence, kv head) are
-    // taken by one workgroup (if the states of all their runs fit into its LDS): the same numbers, one kernel.
-    const bool fold = n_splits > 1 && (long long)n_kv * n_seqs >= compute_units() &&
-                      lds_bytes * n_splits <= DEC_FOLD_LDS;
-    if (fold) {
+    if (mode == DEC_FOLD) {
         lds_bytes *= n_splits;  // a row for every run
         if (lds_bytes > 48 * 1024) {  // beyond the default limit of dynamic LDS
             static bool allowed[64];
@@ -947,13 +994,14 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
             }
         }
     }
-    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_kv, n_seqs, fold ? 1 : n_splits), dim3(DEC_WAVES * SIA_WAVE),
-                       lds_bytes, stream, (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages,
-                       (const bf16_t*)v_pages, block_table, table_width, cu_q, kv_len, ws_acc, ws_ml, (bf16_t*)out,
-                       n_heads, n_kv, ps_log2, scale, window, n_splits, fold ? 1 : 0);
-    if (n_splits > 1 && !fold)
+    const dim3 grid(n_kv, n_seqs, mode == DEC_FOLD ? 1 : mode == DEC_SPREAD ? n_splits * DEC_WAVES : n_splits);
+    hipLaunchKernelGGL(attn_decode_kernel, grid, dim3((mode == DEC_SPREAD ? 1 : DEC_WAVES) * SIA_WAVE),
+                       mode == DEC_SPREAD ? 0 : lds_bytes, stream, (const bf16_t*)q, q_row_stride,
+                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, cu_q, kv_len, ws_acc,
+                       ws_ml, (bf16_t*)out, n_heads, n_kv, ps_log2, scale, window, n_splits, (int)mode);
+    if (mode == DEC_SPREAD || (mode == DEC_PLAIN && n_splits > 1))
         hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_heads, n_seqs), dim3(SIA_WAVE), 0, stream, ws_acc,
-                           ws_ml, cu_q, kv_len, (bf16_t*)out, n_heads, n_splits, window);
+                           ws_ml, cu_q, kv_len, (bf16_t*)out, n_heads, n_splits, window, mode == DEC_SPREAD ? 1 : 0);
     return SIA_LAUNCH_CHECK();
 }
 

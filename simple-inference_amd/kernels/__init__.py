@@ -59,6 +59,7 @@ _ATTN_SIGNATURES = {
     "sia_attn_prefill": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "sia_attn_decode_max_splits": [_c_int, _c_int],
+    "sia_attn_decode_workspace": [_c_int, _c_int, _c_int, _c_int, _c_int],
     "sia_attn_prefill_rows": [],
     "sia_attn_prefill_rows_split": [],
     "sia_attn_prefill_rows_long": [],
@@ -188,6 +189,7 @@ class HipKernels:
             name, sources, defines = attention_library_spec(head_dim)
             lib = build.load_library(name, sources, defines)
             _bind(lib, _ATTN_SIGNATURES)
+            lib.sia_attn_decode_workspace.restype = ctypes.c_longlong
             if lib.sia_attn_mfma_head_dim() != head_dim:
                 raise KernelError(f"library {name} was built for another head size")
             self._attn_libs[head_dim] = lib
@@ -525,10 +527,10 @@ class HipKernels:
             # How many workgroups share a (sequence, kv head) is the kernel's decision, from that sequence's own
             # length; the step's longest possible sequence only sizes the grid and the workspaces.
             max_splits = lib.sia_attn_decode_max_splits(int(ctx.kv_bound or ctx.max_kv_len), window)
-            ws_acc = ws_ml = None
-            if max_splits > 1:
-                ws_acc = torch.empty((n_dec * n_heads * max_splits * head_dim,), dtype=torch.float32, device=qkv.device)
-                ws_ml = torch.empty((n_dec * n_heads * max_splits * 2,), dtype=torch.float32, device=qkv.device)
+            ws_acc, ws_ml = (
+                torch.empty((floats,), dtype=torch.float32, device=qkv.device) if floats else None
+                for floats in (lib.sia_attn_decode_workspace(n_dec, n_heads, n_kv_heads, max_splits, which)
+                               for which in (0, 1)))
             self._check(lib.sia_attn_decode(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), _ptr(ws_acc), _ptr(ws_ml), n_dec, n_heads,
