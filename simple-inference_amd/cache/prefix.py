@@ -1,17 +1,19 @@
 """Reuse of the pages of equal prompt prefixes (what the reference's ``serving/radix_cache.py:30-194`` is for).
 
-A prompt's complete pages form a chain: page ``i`` is identified by its own token ids together with
-the identity of page ``i - 1``.  The cache is a flat table from ``(previous entry, token ids of a page)``
-to an entry that pins one page of the pool (all slabs of it), so a request with an equal prefix takes
-those pages by reference and nothing is copied.  A lookup covers complete pages only and always leaves
-at least one prompt token to run, because the first new token needs logits.
+A prompt's complete pages form a chain, and a chain is known by a running digest: the digest of the
+first ``i`` pages is a hash of the digest of the first ``i - 1`` and the token ids of page ``i``.  The
+cache is one table from digest to the pool page that holds such a prefix's last page of keys and
+values (all slabs of it), pinned in the pool, so a request with an equal prefix takes those pages by
+reference and nothing is copied.  An entry remembers its page's token ids and the digest in front of
+it, and a lookup believes a digest only if both agree, so two chains that happen to hash alike are
+told apart.  A lookup covers complete pages only and always leaves at least one prompt token to run,
+because the first new token needs logits.
 
-What is dropped when admission needs pages, or when the cache outgrows ``capacity``, is the entry that
-ends a chain (nothing continues it) and was used longest ago.  Such entries wait in a heap ordered by
-their last use; the heap is cleaned lazily (an item is believed only if its entry still exists, still
-ends a chain and has not been used since), so a lookup, an insertion and an eviction each cost a few
-heap operations however many pages are cached.  A dropped page stays alive while a request still
-holds it.
+What goes when admission needs pages, or when the cache outgrows ``capacity``, is the entry that ends
+a chain (nothing continues it) and was used longest ago.  Candidates wait in a heap ordered by the
+time of their last use; a heap item is believed only if its entry still exists, still ends a chain
+and has not been used since, so a lookup, an insertion and an eviction each cost a few heap
+operations however many pages are cached.  A page that goes stays alive while a request holds it.
 
 It needs a model whose layers all keep every key (one group, no window) and that has no per-request
 state: a shared page must hold everything a later request needs of the prefix.
@@ -20,21 +22,27 @@ state: a shared page must hold everything a later request needs of the prefix.
 from __future__ import annotations
 
 import heapq
-from typing import Dict, Iterable, List, Optional, Tuple
+from typing import Dict, Iterator, List, Optional, Sequence, Tuple
 
-_ROOT = 0
+_NOTHING = 0          # the digest of the empty prefix
 
 
-class _Entry:
-    __slots__ = ("uid", "page", "before", "edge", "continued_by", "used")
+def _extend(digest: int, ids: Tuple[int, ...]) -> int:
+    """The digest of a prefix one page longer."""
+    return hash((digest, ids)) or 1     # never the digest of the empty prefix
 
-    def __init__(self, uid, page, before, edge, used):
-        self.uid = uid                  # identity of the chain up to and including this page
-        self.page = page
-        self.before = before            # the entry of the page in front (None for a prompt's first page)
-        self.edge = edge                # this entry's key in the table
-        self.continued_by = 0           # entries that have this one in front of them
-        self.used = used                # time of the last lookup or insertion that passed through
+
+class _Held:
+    """One cached page: the last page of the prefix whose digest is its key in the table."""
+
+    __slots__ = ("page", "ids", "front", "heirs", "stamp")
+
+    def __init__(self, page: int, ids: Tuple[int, ...], front: int, stamp: int):
+        self.page = page        # the pool's page
+        self.ids = ids          # its token ids
+        self.front = front      # digest of the prefix without this page
+        self.heirs = 0          # cached pages that continue this prefix
+        self.stamp = stamp      # time of the last lookup or insertion that passed through
 
 
 class PrefixCache:
@@ -46,117 +54,115 @@ class PrefixCache:
         self.pool = cache.groups[0].pool
         self.page_size = cache.page_size
         self.capacity = max_pages
-        self._table: Dict[Tuple[int, Tuple[int, ...]], _Entry] = {}
-        self._ends: List[Tuple[int, int]] = []     # heap of (last use, uid) of entries that may end a chain
-        self._by_uid: Dict[int, _Entry] = {}
-        self._uids = _ROOT
-        self._now = 0
-        self.counters = {"lookups": 0, "lookups_hit": 0, "tokens_reused": 0, "pages_dropped": 0}
+        self._known: Dict[int, _Held] = {}
+        self._ends: List[Tuple[int, int]] = []     # heap of (stamp, digest): entries that may end a chain
+        self._tick = 0
+        self._lookups = self._hits = self._reused = self._dropped = 0
 
     def __len__(self) -> int:
-        return len(self._table)
+        return len(self._known)
 
-    # -- the two ways in -----------------------------------------------------------------
-    def _pages_of(self, tokens, n_tokens: int) -> Iterable[Tuple[int, ...]]:
-        ps = self.page_size
-        return (tuple(tokens[i:i + ps]) for i in range(0, n_tokens - ps + 1, ps))
+    def stats(self) -> Dict[str, int]:
+        held = len(self._known)
+        return {"pages": held, "tokens": held * self.page_size, "lookups": self._lookups,
+                "lookups_hit": self._hits, "tokens_reused": self._reused, "pages_dropped": self._dropped}
 
-    def _use(self, entry: _Entry) -> None:
-        entry.used = self._now
-        if not entry.continued_by:
-            heapq.heappush(self._ends, (entry.used, entry.uid))
-            if len(self._ends) > 4 * len(self._table) + 64:    # mostly stale items: start the heap afresh
-                self._ends = [(e.used, e.uid) for e in self._table.values() if not e.continued_by]
-                heapq.heapify(self._ends)
+    # -- making room ---------------------------------------------------------------------
+    def evict_until_available(self, required_pages: int, protected=()) -> bool:
+        """Lets chain ends go, oldest first and never a ``protected`` page, until the pool has ``required_pages``
+        unpromised pages; False if it cannot get there."""
+        spared = frozenset(protected)
+        while self.pool.n_unpromised < required_pages:
+            if not self._let_oldest_end_go(spared):
+                return False
+        return True
+
+    def clear(self) -> None:
+        for digest in list(self._known):
+            self._unpin(digest)
+        del self._ends[:]
+        self._lookups = self._hits = self._reused = self._dropped = 0
+
+    def _let_oldest_end_go(self, spared) -> bool:
+        passed_over = []
+        gone: Optional[_Held] = None
+        while self._ends and gone is None:
+            stamp, digest = heapq.heappop(self._ends)
+            held = self._known.get(digest)
+            if held is None or held.heirs or held.stamp != stamp:
+                continue                            # stale: gone, continued, or used again since
+            if held.page in spared:
+                passed_over.append((stamp, digest))
+                continue
+            gone = self._unpin(digest)
+        for item in passed_over:
+            heapq.heappush(self._ends, item)
+        if gone is None:
+            return False
+        self._dropped += 1
+        front = self._known.get(gone.front)
+        if front is not None:
+            front.heirs -= 1
+            if front.heirs == 0:                    # it ends a chain now, as old as it is
+                heapq.heappush(self._ends, (front.stamp, gone.front))
+        return True
+
+    def _unpin(self, digest: int) -> _Held:
+        held = self._known.pop(digest)
+        self.pool.unpin(held.page)
+        return held
+
+    # -- looking up and taking in ----------------------------------------------------------
+    def _chain(self, tokens: Sequence[int], n_pages: int) -> Iterator[Tuple[int, int, Tuple[int, ...]]]:
+        """(digest in front, digest, token ids) of each of the first ``n_pages`` pages of ``tokens``."""
+        front, size = _NOTHING, self.page_size
+        for first in range(0, n_pages * size, size):
+            ids = tuple(tokens[first:first + size])
+            digest = _extend(front, ids)
+            yield front, digest, ids
+            front = digest
+
+    def _seen(self, held: _Held, digest: int) -> None:
+        held.stamp = self._tick
+        if held.heirs:
+            return
+        heapq.heappush(self._ends, (held.stamp, digest))
+        if len(self._ends) > 4 * len(self._known) + 64:     # mostly stale items: start the heap afresh
+            self._ends = [(h.stamp, d) for d, h in self._known.items() if not h.heirs]
+            heapq.heapify(self._ends)
 
     def match(self, tokens) -> List[int]:
         """Pages of the longest cached chain that starts ``tokens``, at least one token left over."""
-        self._now += 1
-        self.counters["lookups"] += 1
-        usable = (len(tokens) - 1) // self.page_size * self.page_size
-        found: List[int] = []
-        uid = _ROOT
-        for ids in self._pages_of(tokens, usable):
-            entry = self._table.get((uid, ids))
-            if entry is None:
+        self._tick += 1
+        self._lookups += 1
+        pages: List[int] = []
+        for front, digest, ids in self._chain(tokens, (len(tokens) - 1) // self.page_size):
+            held = self._known.get(digest)
+            if held is None or held.front != front or held.ids != ids:
                 break
-            self._use(entry)
-            found.append(entry.page)
-            uid = entry.uid
-        if found:
-            self.counters["lookups_hit"] += 1
-            self.counters["tokens_reused"] += len(found) * self.page_size
-        return found
+            self._seen(held, digest)
+            pages.append(held.page)
+        if pages:
+            self._hits += 1
+            self._reused += self.page_size * len(pages)
+        return pages
 
     def insert(self, tokens, page_table: List[int]) -> None:
         """Keeps every complete page of ``tokens`` whose keys and values are written; ``page_table[i]`` is the
         pool's page of positions ``i * page_size`` onwards."""
-        self._now += 1
         whole = len(tokens) // self.page_size
-        if len(page_table) < whole:
+        if whole > len(page_table):
             raise ValueError(f"{whole} complete pages of tokens, but a table of {len(page_table)} pages")
-        before: Optional[_Entry] = None
-        for i, ids in enumerate(self._pages_of(tokens, whole * self.page_size)):
-            edge = (before.uid if before else _ROOT, ids)
-            entry = self._table.get(edge)
-            if entry is None:
+        self._tick += 1
+        for i, (front, digest, ids) in enumerate(self._chain(tokens, whole)):
+            held = self._known.get(digest)
+            if held is not None and (held.front != front or held.ids != ids):
+                break             # another chain with this digest is cached: this one stays out from here on
+            if held is None:
                 self.pool.pin(page_table[i])      # raises for a page that nobody holds: nothing is recorded then
-                self._uids += 1
-                entry = _Entry(self._uids, page_table[i], before, edge, self._now)
-                self._table[edge] = self._by_uid[entry.uid] = entry
-                if before is not None:
-                    before.continued_by += 1
-            self._use(entry)
-            before = entry
-        while len(self._table) > self.capacity and self._drop_oldest_end(()):
+                held = self._known[digest] = _Held(page_table[i], ids, front, self._tick)
+                if front != _NOTHING:
+                    self._known[front].heirs += 1
+            self._seen(held, digest)
+        while len(self._known) > self.capacity and self._let_oldest_end_go(frozenset()):
             pass
-
-    # -- the way out ---------------------------------------------------------------------
-    def evict_until_available(self, required_pages: int, protected=()) -> bool:
-        """Drops chain ends, oldest first and never a ``protected`` page, until the pool has ``required_pages``
-        unpromised pages; False if it cannot get there."""
-        protected = frozenset(protected)
-        while self.pool.n_unpromised < required_pages:
-            if not self._drop_oldest_end(protected):
-                return False
-        return True
-
-    def _drop_oldest_end(self, protected) -> bool:
-        spared = []
-        victim = None
-        while self._ends:
-            used, uid = heapq.heappop(self._ends)
-            entry = self._by_uid.get(uid)
-            if entry is None or entry.continued_by or entry.used != used:
-                continue                          # stale: dropped, continued or used again since
-            if entry.page in protected:
-                spared.append((used, uid))
-                continue
-            victim = entry
-            break
-        for item in spared:
-            heapq.heappush(self._ends, item)
-        if victim is None:
-            return False
-        self._forget(victim)
-        self.counters["pages_dropped"] += 1
-        if victim.before is not None:
-            victim.before.continued_by -= 1
-            if not victim.before.continued_by:    # it ends a chain now, with the age it has
-                heapq.heappush(self._ends, (victim.before.used, victim.before.uid))
-        return True
-
-    def _forget(self, entry: _Entry) -> None:
-        del self._table[entry.edge]
-        del self._by_uid[entry.uid]
-        self.pool.unpin(entry.page)
-
-    def clear(self) -> None:
-        for entry in list(self._table.values()):
-            self._forget(entry)
-        self._ends.clear()
-        for key in self.counters:
-            self.counters[key] = 0
-
-    def stats(self) -> Dict[str, int]:
-        return {"pages": len(self._table), "tokens": len(self._table) * self.page_size, **self.counters}

@@ -20,22 +20,88 @@ sketches it).
 from __future__ import annotations
 
 from collections import deque
-from typing import Callable, Deque, List, Optional, Tuple
+from typing import Callable, Deque, Iterator, List, Optional, Tuple
 
 from .request import Request, RequestState
 
 Gate = Optional[Callable[[Request], bool]]
+Share = Tuple[Request, int]      # a request and the number of its next tokens that a step runs
 
 
 class Scheduler:
     def __init__(self, max_running: int, token_budget: int, chunk_tokens: int):
-        if max_running <= 0 or chunk_tokens <= 0:
-            raise ValueError("max_running and chunk_tokens must be positive")
-        self.max_running = max_running
-        self.token_budget = token_budget
-        self.chunk_tokens = chunk_tokens
+        for name, value in (("max_running", max_running), ("chunk_tokens", chunk_tokens)):
+            if value <= 0:
+                raise ValueError(f"{name} must be positive, got {value}")
+        self.max_running, self.token_budget, self.chunk_tokens = max_running, token_budget, chunk_tokens
         self.queue: Deque[Request] = deque()     # not yet let in, oldest first
         self.live: List[Request] = []            # let in and not yet retired, in the order they came in
+
+    # -- one step ------------------------------------------------------------------------
+    def plan(self, gate: Gate = None, admit: bool = True) -> List[Share]:
+        """The shares of one step: decoded tokens first, then prompt portions, then the first portions of requests
+        that come in with this step (none with ``admit`` False)."""
+        room = self.chunk_tokens
+        shares: List[Share] = []
+        for req in self._in_state(RequestState.DECODE):
+            shares.append((req, 1))
+            room -= 1
+        sources = [self._in_state(RequestState.PREFILL)]
+        if admit:
+            sources.append(self._newcomers(gate))
+        for source in sources:
+            while room > 0:     # asked before the next request is: nobody comes in for nothing
+                req = next(source, None)
+                if req is None:
+                    break
+                n = req.tokens_wanted(room)
+                shares.append((req, n))
+                room -= n
+        return shares
+
+    def _in_state(self, state: RequestState) -> Iterator[Request]:
+        return (req for req in self.live if req.state is state)
+
+    def _newcomers(self, gate: Gate) -> Iterator[Request]:
+        """Requests as they come in, for as long as the head of the queue may (asked for one at a time: nobody comes
+        in whom the step has no room for)."""
+        while True:
+            req = self.let_in(gate)
+            if req is None:
+                return
+            yield req
+
+    # -- coming and going ------------------------------------------------------------------
+    def let_in(self, gate: Gate = None) -> Optional[Request]:
+        """The head of the queue comes in if slot, budget and ``gate`` allow; returns it, or None.  ``gate`` is
+        expected to give the request its slot and pages (``Request.enter``); without one it just turns to PREFILL."""
+        head = self.queue[0] if self.queue else None
+        if head is None or not self._has_room_for(head) or not (gate is None or gate(head)):
+            return None
+        self.live.append(self.queue.popleft())
+        if head.state is RequestState.WAITING:
+            head.state = RequestState.PREFILL
+        return head
+
+    def _has_room_for(self, newcomer: Request) -> bool:
+        if len(self.live) >= self.max_running:
+            return False
+        if not self.live:
+            return True             # an empty engine takes any one request, however long
+        inside = 0
+        for req in self.live:
+            inside += req.context_len
+        return inside + newcomer.prompt_len <= self.token_budget
+
+    def retire(self) -> List[Request]:
+        """Takes the finished requests out; returns them."""
+        staying: List[Request] = []
+        gone: List[Request] = []
+        for req in self.live:
+            (gone if req.state is RequestState.FINISHED else staying).append(req)
+        if gone:
+            self.live = staying
+        return gone
 
     def submit(self, req: Request) -> None:
         if req.state is not RequestState.WAITING:
@@ -43,55 +109,11 @@ class Scheduler:
         self.queue.append(req)
 
     def busy(self) -> bool:
-        return bool(self.queue) or bool(self.live)
+        return len(self.queue) + len(self.live) > 0
 
     def clear(self) -> None:
         self.queue.clear()
-        self.live.clear()
-
-    def retire(self) -> List[Request]:
-        """Takes the finished requests out; returns them."""
-        gone = [r for r in self.live if r.state is RequestState.FINISHED]
-        if gone:
-            self.live = [r for r in self.live if r.state is not RequestState.FINISHED]
-        return gone
-
-    def let_in(self, gate: Gate = None) -> Optional[Request]:
-        """The head of the queue comes in if slot, budget and ``gate`` allow; returns it, or None.  ``gate`` is
-        expected to give the request its slot and pages (``Request.enter``); without one it just turns to PREFILL."""
-        if not self.queue or len(self.live) >= self.max_running:
-            return None
-        head = self.queue[0]
-        if self.live and sum(r.context_len for r in self.live) + head.prompt_len > self.token_budget:
-            return None
-        if gate is not None and not gate(head):
-            return None
-        self.queue.popleft()
-        if head.state is RequestState.WAITING:
-            head.state = RequestState.PREFILL
-        self.live.append(head)
-        return head
-
-    def plan(self, gate: Gate = None, admit: bool = True) -> List[Tuple[Request, int]]:
-        """(request, number of its next tokens) for one step: decoded tokens first, then prompt portions, then the
-        first portions of requests that come in with this step (none with ``admit`` False)."""
-        step: List[Tuple[Request, int]] = [(r, 1) for r in self.live if r.state is RequestState.DECODE]
-        room = self.chunk_tokens - len(step)
-        for r in self.live:
-            if room <= 0:
-                break
-            if r.state is RequestState.PREFILL:
-                n = r.tokens_wanted(room)
-                step.append((r, n))
-                room -= n
-        while admit and room > 0:
-            newcomer = self.let_in(gate)
-            if newcomer is None:
-                break
-            n = newcomer.tokens_wanted(room)
-            step.append((newcomer, n))
-            room -= n
-        return step
+        del self.live[:]
 
     def __repr__(self) -> str:
         return f"<scheduler: {len(self.queue)} queued, {len(self.live)} of {self.max_running} slots live>"
