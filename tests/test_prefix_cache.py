@@ -96,6 +96,27 @@ def test_the_lazy_heap_is_started_afresh_when_it_is_mostly_stale():
     assert pc.evict_until_available(4) and m.free_pages() == 4
 
 
+def test_chains_whose_digests_collide_are_told_apart(monkeypatch):
+    """A prefix is known by a digest of its pages; an entry also keeps its page's ids and the digest in front, and a
+    lookup believes a digest only if both agree.  With a digest that is the same for everything, nothing is ever
+    found that was not put in: the first page of the first prompt is cached, whatever collides with it stays out."""
+    from simple_inference_amd.cache import prefix
+    monkeypatch.setattr(prefix, "_extend", lambda digest, ids: 7)
+    m = manager(8)
+    pc = PrefixCache(m, max_pages=8)
+    for rid, toks in ((1, [1, 2, 3, 4]), (2, [5, 6, 7, 8])):
+        m.admit(rid, total_tokens=4)
+        m.extend(rid, 4)
+        pc.insert(toks, m.table(0, rid))
+    assert len(pc) == 1
+    assert pc.match([1, 2, 3, 4, 0]) == m.table(0, 1)[:1]      # its second page has the digest of its first
+    assert pc.match([5, 6, 7, 8, 0]) == [] and pc.match([3, 4, 0]) == []
+    m.release(1)
+    m.release(2)
+    assert pc.evict_until_available(8) and len(pc) == 0
+    m.check()
+
+
 def test_refuses_models_it_cannot_serve():
     with pytest.raises(ValueError, match="window"):
         PrefixCache(manager(4, window=8), max_pages=4)
