@@ -945,7 +945,9 @@ static DecodeMode decode_mode(int n_seqs, int n_heads, int n_kv, int max_splits)
     const long long pairs = (long long)n_kv * n_seqs, cus = compute_units();
     const size_t row_bytes = (size_t)(n_heads / n_kv) * (HD + 2) * sizeof(float);
     if (max_splits > 1 && pairs >= cus && DEC_WAVES * row_bytes * max_splits <= (size_t)DEC_FOLD_LDS) return DEC_FOLD;
-    if (pairs * max_splits <= cus) return DEC_SPREAD;  // no more splits than compute units: a workgroup for every run
+    // no more splits than compute units: a workgroup for every run.  Not for sequences too short to split: their one
+    // workgroup writes the result itself, which costs less than a second kernel that merges runs.
+    if (max_splits > 1 && pairs * max_splits <= cus) return DEC_SPREAD;
     return DEC_PLAIN;
 }
 
