@@ -564,9 +564,12 @@ class HipKernels:
             self._want(top_p, "top_p", torch.float32, (rows,))
             self._want(uniform, "uniform", torch.float32, (rows,))
         out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-        # the histograms of the filters start at zero; an argmax-only call reads nothing that it has not written
-        make = torch.zeros if filters else torch.empty
-        workspace = make((self.core.sia_sample_workspace_bytes(rows),), dtype=torch.uint8, device=logits.device)
+        # One workspace, kept and grown as needed: the kernels set to zero what they need at zero, and calls follow
+        # one another on the stream.  (Callers on several streams at once need a kernels object each.)
+        need = self.core.sia_sample_workspace_bytes(rows)
+        workspace = getattr(self, "_sample_workspace", None)
+        if workspace is None or workspace.numel() < need or workspace.device != logits.device:
+            workspace = self._sample_workspace = torch.empty((need,), dtype=torch.uint8, device=logits.device)
         self._check(self.core.sia_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
                                          _ptr(out), _ptr(workspace), rows, vocab, filters, self._stream()), "sample")
         return out

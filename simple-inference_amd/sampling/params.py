@@ -11,6 +11,9 @@ of the request's ``seed`` and n.
 from __future__ import annotations
 
 from dataclasses import dataclass
+from typing import Sequence
+
+import numpy as np
 
 _MASK = (1 << 64) - 1
 
@@ -48,3 +51,18 @@ def uniform_for(seed: int, draw_index: int) -> float:
     """The uniform number in [0, 1) of a request's ``draw_index``-th draw (24 bits, exact in float32)."""
     h = _splitmix64(_splitmix64(seed & _MASK) ^ ((draw_index + 1) * 0xD6E8FEB86659FD93 & _MASK))
     return (h >> 40) / float(1 << 24)
+
+
+def _splitmix64_each(x: np.ndarray) -> np.ndarray:
+    x = x + np.uint64(0x9E3779B97F4A7C15)          # unsigned 64-bit arrays wrap around, as the masks above do
+    x = (x ^ (x >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+    x = (x ^ (x >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    return x ^ (x >> np.uint64(31))
+
+
+def uniforms_for(seeds: Sequence[int], draw_indices: Sequence[int]) -> np.ndarray:
+    """``uniform_for`` of each (seed, draw index), as float32: the same numbers, computed for a whole batch at once."""
+    seed = np.array([s & _MASK for s in seeds], dtype=np.uint64)
+    draw = np.array([(n + 1) & _MASK for n in draw_indices], dtype=np.uint64)
+    h = _splitmix64_each(_splitmix64_each(seed) ^ (draw * np.uint64(0xD6E8FEB86659FD93)))
+    return ((h >> np.uint64(40)).astype(np.float32)) / np.float32(1 << 24)
