@@ -733,10 +733,20 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     scale *= LOG2E;  // exponentials are taken as powers of two
     const int n_blocks = gridDim.x * gridDim.y;
     int vid = blockIdx.y * gridDim.x + blockIdx.x;
-    if (n_blocks % 8 == 0) vid = (vid % 8) * (n_blocks / 8) + vid / 8;
-    const int head = vid / gridDim.x;
+    int head, tile;
+    if (n_heads % 8 == 0) {
+        // a die's heads take turns tile by tile, so that on every die the workgroups with most keys (see below)
+        // start first and the short ones fill the compute units up at the end
+        const int heads_here = n_heads / 8, die = vid % 8, turn = vid / 8;
+        head = die * heads_here + turn % heads_here;
+        tile = turn / heads_here;
+    } else {
+        if (n_blocks % 8 == 0) vid = (vid % 8) * (n_blocks / 8) + vid / 8;
+        head = vid / gridDim.x;
+        tile = vid % gridDim.x;
+    }
     // which sequence and which of its row tiles this workgroup has; late tiles (most keys) come first
-    int tile = vid % gridDim.x, seq = seq_begin;
+    int seq = seq_begin;
     for (; seq < seq_end; ++seq) {
         const int tiles = (cu_q[seq + 1] - cu_q[seq] + ROWS - 1) / ROWS;
         if (tile < tiles) {
@@ -1051,16 +1061,16 @@ SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_p
         return launch_prefill<1, PF_ROWS / 16, 1>(n_tiles, ARGS);
     } else {
         // Which shape is the fastest follows the number of workgroups per compute unit (measured at 24 heads of 128
-        // on 256 compute units): the split shape while all its workgroups are on the chip at once (under 5/8 of a
-        // wide workgroup per compute unit: prompts or portions up to about 800 tokens), the paired shape of 128
+        // on 256 compute units): the split shape while all its workgroups are on the chip at once (up to 6/8 of a
+        // wide workgroup per compute unit: prompts or portions up to about 1,000 tokens), the paired shape of 128
         // tokens (two tiles of keys a step, one for each set of waves) up to 15/8 (about 2,500 tokens), the wide
-        // shape (one tile a step) beyond, and from 75/8 on (about 12,000 tokens) 8 waves of 32 tokens (256 tokens a
+        // shape (one tile a step) beyond, and from 36/8 on (about 6,000 tokens) 8 waves of 32 tokens (256 tokens a
         // workgroup, two tiles a step: a tile staged in LDS then serves twice as many tokens).
         const long long wide_groups = (long long)n_tiles * n_heads, cus = compute_units();
-        if (PF_USE_LDS && n_tiles_split > 0 && wide_groups * 8 <= cus * 5)
+        if (PF_USE_LDS && n_tiles_split > 0 && wide_groups * 8 <= cus * 6)
             return launch_prefill<1, 2 * PF_ROWS_SPLIT / 16, 2>(n_tiles_split, ARGS);
         if (PF_USE_LDS && wide_groups * 8 <= cus * 15) return launch_prefill<2, 2 * PF_ROWS / 32, 2, 2>(n_tiles, ARGS);
-        if (PF_USE_LDS && n_tiles_long > 0 && wide_groups * 8 >= cus * 75)
+        if (PF_USE_LDS && n_tiles_long > 0 && wide_groups * 8 >= cus * 36)
             return launch_prefill<2, PF_ROWS_LONG / 32, 1, 2>(n_tiles_long, ARGS);
         return launch_prefill<2, PF_ROWS / 32, 1>(n_tiles, ARGS);
     }

@@ -61,9 +61,12 @@ class StepRunner:
                 raise ValueError(
                     f"request {e.req} would reach position {self.cache.lengths[e.req] + len(e.tokens)}, "
                     f"beyond the engine's {self.max_positions}")
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise ValueError(f"token id {t} of request {e.req} is outside [0, {self.vocab_size})")
+            ids = np.asarray(e.tokens)      # checked as a whole: a prompt portion has thousands
+            if ids.dtype.kind not in "iu":
+                raise ValueError(f"the token ids of request {e.req} are not integers ({ids.dtype})")
+            if int(ids.min()) < 0 or int(ids.max()) >= self.vocab_size:
+                t = next(int(t) for t in ids if not 0 <= int(t) < self.vocab_size)
+                raise ValueError(f"token id {t} of request {e.req} is outside [0, {self.vocab_size})")
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"wanted place {w} of request {e.req} is outside its {len(e.tokens)} tokens")

@@ -639,6 +639,28 @@ def test_sample_filters_at_their_edges(hip, vocab):
     assert hip.sample(*args, filters=0).tolist() == hip.sample(*args).tolist() == twin.sample(*args).tolist()
 
 
+def test_sample_does_not_care_what_its_workspace_held(hip):
+    """The sampler sets to zero what it needs at zero: a workspace full of ones gives the tokens of a zeroed one,
+    and the kernels object's own workspace, used by every call before this one, gives them too."""
+    rows, vocab = 6, 3001
+    logits = rnd(rows, vocab, seed=8, scale=2.5)
+    temperature = torch.tensor([0.9, 0.0, 1.1, 0.6, 1.0, 0.8], dtype=torch.float32, device=DEV)
+    top_k = torch.tensor([40, 0, 0, 7, 0, 2999], dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([0.9, 1.0, 0.6, 1.0, 1.0, 0.95], dtype=torch.float32, device=DEV)
+    u = torch.tensor([0.11, 0.5, 0.93, 0.42, 0.77, 0.3], dtype=torch.float32, device=DEV)
+    want = hip.sample(logits, temperature, top_k, top_p, u).tolist()
+    assert want == twin.sample(logits, temperature, top_k, top_p, u).tolist()
+    size = hip.core.sia_sample_workspace_bytes(rows)
+    for fill in (0, 255, 1):
+        out = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        workspace = torch.full((size,), fill, dtype=torch.uint8, device=DEV)
+        code = hip.core.sia_sample(logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
+                                   u.data_ptr(), out.data_ptr(), workspace.data_ptr(), rows, vocab, 7,
+                                   torch.cuda.current_stream().cuda_stream)
+        assert code == 0
+        assert out.tolist() == want, fill
+
+
 @pytest.mark.parametrize("vocab", [5, 1001, 4096, 128256])
 def test_argmax_of_all_greedy_steps(hip, vocab):
     rows = 9
