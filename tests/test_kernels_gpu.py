@@ -247,6 +247,29 @@ def test_rope_kv_write_and_attention(hip, dtype, geom):
         torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("geom", [(24, 8, 128, 128, 16), (5, 1, 48, 32, 8), (3, 3, 64, 64, 4)])
+def test_rope_kv_write_of_a_long_step(hip, geom):
+    """More than a thousand tokens in one step (the kernel then gives a thread several items): two prompt portions,
+    one from the start of its sequence and one that begins in the middle of a page, and a single decoded token."""
+    n_heads, n_kv, D, rd, ps = geom
+    q_lens, kv_lens = [1, 700, 450], [77, 700, 450 + 21]
+    ctx = Ctx(q_lens, kv_lens)
+    pages = sum(-(-kv // ps) for kv in kv_lens) + 2
+    c_hip = Cache(pages, n_kv, ps, D, torch.bfloat16, kv_lens, seed=14)
+    c_twin = Cache(pages, n_kv, ps, D, torch.bfloat16, kv_lens, seed=14)
+    c_hip.k_pages.copy_(rnd(*c_hip.k_pages.shape, dtype=torch.bfloat16, seed=15)); c_twin.k_pages.copy_(c_hip.k_pages)
+    c_hip.v_pages.copy_(rnd(*c_hip.v_pages.shape, dtype=torch.bfloat16, seed=16)); c_twin.v_pages.copy_(c_hip.v_pages)
+    qkv = rnd(ctx.n_tokens, (n_heads + 2 * n_kv) * D, dtype=torch.bfloat16, seed=17)
+    q1, q2 = qkv.clone(), qkv.clone()
+    ang = torch.outer(torch.arange(720, dtype=torch.float32), 1.0 / (500000.0 ** (torch.arange(0, rd, 2, dtype=torch.float32) / rd)))
+    cos, sin = ang.cos().to(DEV), ang.sin().to(DEV)
+    hip.rope_kv_write(q1, n_heads, n_kv, D, rd, cos, sin, ctx, c_hip)
+    twin.rope_kv_write(q2, n_heads, n_kv, D, rd, cos, sin, ctx, c_twin)
+    torch.testing.assert_close(q1.float(), q2.float(), **tol(torch.bfloat16))
+    torch.testing.assert_close(c_hip.k_pages.float(), c_twin.k_pages.float(), **tol(torch.bfloat16))
+    assert torch.equal(c_hip.v_pages, c_twin.v_pages)
+
+
 @pytest.mark.parametrize("geom", [
     # heads, kv heads, head_dim, page_size, hidden, rows
     (24, 8, 128, 64, 3072, 8), (3, 1, 32, 8, 192, 16), (5, 5, 96, 16, 1088, 1), (2, 1, 256, 32, 64, 5),
