@@ -41,6 +41,25 @@ class StepRunner:
         self.device = torch.device(device)
         self.max_positions = max_positions
         self.vocab_size = model.vocab_size
+        self._stages, self._stage_turn = [], -1
+
+    def _staging(self, size: int):
+        """Host memory for a step's metadata: on a GPU one of a few pinned buffers used in turn (each free again when
+        the copy out of it has run), so that the host can lay out the next step while earlier ones are still queued."""
+        if self.device.type != "cuda":
+            return np.empty(size, dtype=np.int32), None
+        self._stage_turn = (self._stage_turn + 1) % 3
+        if len(self._stages) <= self._stage_turn:
+            self._stages.append(None)
+        stage = self._stages[self._stage_turn]
+        if stage is None or stage[0].numel() < size:
+            pinned = torch.empty(max(size, 4096, 2 * (stage[0].numel() if stage else 0)), dtype=torch.int32, pin_memory=True)
+            stage = self._stages[self._stage_turn] = (pinned, torch.cuda.Event(), [False])
+        pinned, copied, used = stage
+        if used[0]:
+            copied.synchronize()    # long done, unless the host is three steps ahead
+        used[0] = True
+        return pinned.numpy()[:size], (pinned, copied)
 
     def _check(self, entries: List[StepEntry]) -> None:
         seen = set()
@@ -100,7 +119,7 @@ class StepRunner:
         sizes = [n_tokens, n_tokens, n_tokens, n_seqs + 1, n_seqs, n_seqs, max(n_rows, 1)] + \
                 [n_seqs * width] * n_groups + [n_moved, n_moved] + [n_tokens] * len(extra_keys)
         offsets = np.concatenate([[0], np.cumsum(sizes)])
-        host = np.empty(int(offsets[-1]), dtype=np.int32)
+        host, staged = self._staging(int(offsets[-1]))
         tok, pos, sot, cu, kvl, slots, rows = (host[offsets[i]:offsets[i + 1]] for i in range(7))
         cu[0] = 0
         rows[:] = 0
@@ -140,7 +159,13 @@ class StepRunner:
                 col[t:t + len(e.tokens)] = e.extra[key]
                 t += len(e.tokens)
 
-        dev = torch.from_numpy(host).to(self.device)
+        if staged is None:
+            dev = torch.from_numpy(host).to(self.device)
+        else:   # from pinned memory, without waiting for the steps that are still queued in front of this one
+            pinned, copied = staged
+            dev = torch.empty(host.size, dtype=torch.int32, device=self.device)
+            dev.copy_(pinned[:host.size], non_blocking=True)
+            copied.record()
         part = lambda i: dev[int(offsets[i]):int(offsets[i + 1])]
         if n_moved:
             self.kernels.place_tokens(part(0), part(7 + n_groups), device_tokens, part(8 + n_groups))
