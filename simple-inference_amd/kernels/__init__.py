@@ -517,31 +517,52 @@ class HipKernels:
             self._stream()), "attention_generic")
         return out
 
-    def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
-        lib = self._attn_lib(head_dim)
-        width = qkv.shape[1]
-        table = cache.block_table
+    def _attention_plan(self, lib, device, n_heads, n_kv_heads, head_dim, window, ctx):
+        """What the attention launches of a step need beside the tensors: the same for every layer with this
+        geometry, so it is worked out once per step and kept with the step's context (workspaces included: a step's
+        layers run one after the other)."""
+        key = (n_heads, n_kv_heads, head_dim, window)
+        plans = getattr(ctx, "attention_plans", None)
+        if plans is not None and key in plans:
+            return plans[key]
         group = n_heads // n_kv_heads
         n_dec = ctx.n_decode_seqs if group <= 16 and 4 * group * (head_dim + 2) * 4 <= 65536 else 0
+        max_splits, ws_acc, ws_ml = 1, None, None
         if n_dec:
             # How many workgroups share a (sequence, kv head) is the kernel's decision, from that sequence's own
             # length; the step's longest possible sequence only sizes the grid and the workspaces.
             max_splits = lib.sia_attn_decode_max_splits(int(ctx.kv_bound or ctx.max_kv_len), window)
             ws_acc, ws_ml = (
-                torch.empty((floats,), dtype=torch.float32, device=qkv.device) if floats else None
+                torch.empty((floats,), dtype=torch.float32, device=device) if floats else None
                 for floats in (lib.sia_attn_decode_workspace(n_dec, n_heads, n_kv_heads, max_splits, which)
                                for which in (0, 1)))
+        tiles = (0, 0, 0)
+        if n_dec < ctx.n_seqs:
+            tiles = tuple(sum(-(-q // rows) for q in ctx.q_lens[n_dec:]) if rows else 0
+                          for rows in (lib.sia_attn_prefill_rows(), lib.sia_attn_prefill_rows_split(),
+                                       lib.sia_attn_prefill_rows_long()))
+        plan = (n_dec, max_splits, ws_acc, ws_ml, tiles)
+        if plans is None:
+            try:
+                ctx.attention_plans = plans = {}
+            except AttributeError:      # a context that takes no further attributes: nothing is kept
+                return plan
+        plans[key] = plan
+        return plan
+
+    def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
+        lib = self._attn_lib(head_dim)
+        width = qkv.shape[1]
+        table = cache.block_table
+        n_dec, max_splits, ws_acc, ws_ml, (n_tiles, n_tiles_split, n_tiles_long) = self._attention_plan(
+            lib, qkv.device, n_heads, n_kv_heads, head_dim, window, ctx)
+        if n_dec:
             self._check(lib.sia_attn_decode(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), _ptr(ws_acc), _ptr(ws_ml), n_dec, n_heads,
                 n_kv_heads, cache.page_size, float(scale), window, max_splits, self._stream()),
                 "attn_decode")
         if n_dec < ctx.n_seqs:
-            rows, rows_split = lib.sia_attn_prefill_rows(), lib.sia_attn_prefill_rows_split()
-            n_tiles = sum(-(-q // rows) for q in ctx.q_lens[n_dec:])
-            n_tiles_split = sum(-(-q // rows_split) for q in ctx.q_lens[n_dec:]) if rows_split else 0
-            rows_long = lib.sia_attn_prefill_rows_long()
-            n_tiles_long = sum(-(-q // rows_long) for q in ctx.q_lens[n_dec:]) if rows_long else 0
             self._check(lib.sia_attn_prefill(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_tiles_split, n_tiles_long, n_heads,
