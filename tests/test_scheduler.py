@@ -1,12 +1,14 @@
 """The scheduler's decisions and the engine around it, on the CPU with the torch twins of the kernels."""
 
+import random
+
 import pytest
 
 import plain_llama as plain
 from helpers import TINIES, random_tokens, write_tiny_model
 from simple_inference_amd import Engine, EngineConfig, RequestState, SamplingParams
 from simple_inference_amd.engine import Request, Scheduler
-from simple_inference_amd.sampling import uniform_for
+from simple_inference_amd.sampling import uniform_for, uniforms_for
 from twins import TwinKernels
 
 
@@ -219,6 +221,18 @@ def test_temperature_sampling_is_seeded_per_request_and_independent_of_the_batch
         eng.run()
         assert [r.generated for r in reqs] == want, kw
     assert len({tuple(t) for t in want}) == 4
+
+
+def test_a_batch_of_uniform_numbers_is_the_numbers_one_by_one():
+    """The sampler computes a step's uniform numbers for all its rows at once: bit for bit what ``uniform_for`` gives
+    for each (seed, draw), also for seeds that are negative or wider than 64 bits, and all in [0, 1)."""
+    rng = random.Random(5)
+    seeds = [0, 1, -1, -12345, 2 ** 63, 2 ** 64 - 1, 2 ** 64, 2 ** 70 + 3] + [rng.getrandbits(64) for _ in range(100)]
+    draws = [0, 1, 2, 2 ** 31, 2 ** 63, 7, 10 ** 6, 3] + [rng.randrange(10 ** 6) for _ in range(100)]
+    batch = uniforms_for(seeds, draws)
+    assert batch.dtype.name == "float32" and batch.shape == (len(seeds),)
+    assert [float(u) for u in batch] == [uniform_for(s, n) for s, n in zip(seeds, draws)]
+    assert all(0.0 <= float(u) < 1.0 for u in batch)
 
 
 def test_stops_at_eos_and_generate_does_not_yield_it(folder):
