@@ -17,8 +17,8 @@
 //      of the floats, 11 + 11 + 10 bits, one counting pass per digit;
 //   3. top-p: the lowest kept value the same way, with the probability mass per digit in place of
 //      the count;
-//   4. one workgroup per row walks the row once for the mass of what is kept, piece by piece in index order, and
-//      once more through the piece in which the cumulative mass passes u * total.
+//   4. the mass of what is kept, for SP_PIECES pieces of consecutive tokens of the row (a piece a wave), and then
+//      one wave per row that finds the piece in which the cumulative mass passes u * total and the token in it.
 // Probabilities enter every sum as fixed-point integers (exp(x - max) * 2^s with the largest s that keeps
 // a row's sum below 2^63: 46 bits for 128,256 entries): integer sums do not depend on their order, so
 // histograms can be built with atomics and every workgroup that recomputes a sum gets the same bits.  A
