@@ -177,8 +177,16 @@ class Engine:
             launched = self._launch(None)
             if launched is None:
                 return {}
-        if self._next_step_is_certain(launched[0]):
-            self._ahead = self._launch(launched)   # before the host waits for this step's tokens
+        if self.cfg.run_ahead and launched[0]:
+            # The next step is planned before the host waits for this one's tokens.  What it needs to know of them it
+            # knows already: a request whose token in flight is its last by count ends now, as far as planning goes
+            # (its pages and slot go back: the next step follows this one on the stream, so whoever gets them
+            # writes them after this step has read them).  An end-of-sequence token is found out a step late.
+            for req in launched[0]:
+                if req.last_token_is_in_flight():
+                    req.end_ahead()
+                    self.cache.release(req.id)
+            self._ahead = self._launch(launched)
         return self._collect(*launched)
 
     def _launch(self, before):
@@ -269,15 +277,9 @@ class Engine:
             for req, token in zip(emitters, tokens[1]()):
                 if req.deliver(int(token), self.eos_ids):
                     emitted[req.id] = int(token)
-                    if req.state is RequestState.FINISHED:
-                        self.cache.release(req.id)
+                    if req.state is RequestState.FINISHED and req.id in self.cache.lengths:
+                        self.cache.release(req.id)      # unless it went back when the request ended ahead
         return emitted
-
-    def _next_step_is_certain(self, emitters: List[Request]) -> bool:
-        """True if the step after the one whose tokens are still on the device can be planned without them: none
-        of its requests reaches ``max_new_tokens`` with the token it is about to get.  (An end-of-sequence token
-        is found out a step late.)"""
-        return bool(self.cfg.run_ahead and emitters) and all(r.length_is_certain_after_next_token() for r in emitters)
 
     def run(self) -> Dict[int, Request]:
         """Steps until every queued request has finished; returns them by id."""

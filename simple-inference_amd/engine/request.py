@@ -21,6 +21,7 @@ class RequestState(enum.Enum):
     WAITING = "waiting"
     PREFILL = "prefill"
     DECODE = "decode"
+    ENDING = "ending"        # its last token is sampled but not read yet; pages and slot are given back already
     FINISHED = "finished"
 
 
@@ -72,6 +73,11 @@ class Request:
         known once the token has been read)."""
         return len(self.generated) + self.in_flight < self.params.max_new_tokens
 
+    def last_token_is_in_flight(self) -> bool:
+        """True if the token that has been sampled for it and not read yet is its last by count, whatever it is."""
+        return (self.state is RequestState.DECODE and self.in_flight > 0
+                and len(self.generated) + self.in_flight >= self.params.max_new_tokens)
+
     # -- transitions ---------------------------------------------------------------------
     def enter(self, slot: int, reused_tokens: int = 0) -> None:
         """Admitted: it has a slot, and ``reused_tokens`` of its prompt are in the cache already."""
@@ -101,6 +107,14 @@ class Request:
         self.state = RequestState.DECODE
         self.in_flight += 1
         self.in_flight_row = row
+
+    def end_ahead(self) -> None:
+        """Its last token is in flight: it takes part in no later step and holds nothing any more; ``deliver`` ends
+        it when the token is read."""
+        if not self.last_token_is_in_flight():
+            raise ValueError(f"request {self.id} cannot end before its tokens are read: {self!r}")
+        self.state = RequestState.ENDING
+        self.slot = None
 
     def deliver(self, token: int, eos_ids=()) -> bool:
         """The host has read a sampled token.  False if the request had ended before (the token was sampled a step

@@ -94,11 +94,11 @@ class Scheduler:
         return inside + newcomer.prompt_len <= self.token_budget
 
     def retire(self) -> List[Request]:
-        """Takes the finished requests out; returns them."""
+        """Takes out the requests that have finished, or will with a token that is sampled already; returns them."""
         staying: List[Request] = []
         gone: List[Request] = []
         for req in self.live:
-            (gone if req.state is RequestState.FINISHED else staying).append(req)
+            (gone if req.state in (RequestState.FINISHED, RequestState.ENDING) else staying).append(req)
         if gone:
             self.live = staying
         return gone

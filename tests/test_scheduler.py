@@ -169,13 +169,20 @@ def test_tokens_do_not_depend_on_batching_queueing_or_portions(folder):
         eng.cache.check()
 
 
-def test_a_request_that_finds_no_pages_waits_for_a_finished_one(folder):
-    """serving/test_paged_kv_cache.py:247-269: 2 pages, two 3-token prompts with 1 new token each."""
-    eng = engine(folder, block_size=4, num_kv_blocks=1, max_running=2)
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_a_request_that_finds_no_pages_waits_for_a_finished_one(folder, run_ahead):
+    """serving/test_paged_kv_cache.py:247-269: 2 pages, two 3-token prompts with 1 new token each.  Running ahead,
+    the engine knows that the first request's one token is its last before it has read it: the second request gets
+    the page in the same call, and its step is on its way when the call returns."""
+    eng = engine(folder, block_size=4, num_kv_blocks=1, max_running=2, run_ahead=run_ahead)
     a = eng.add_request([1, 4, 6], max_new_tokens=1)
     b = eng.add_request([1, 5, 9], max_new_tokens=1)
     eng.step()
-    assert a.state is RequestState.FINISHED and b.state is RequestState.WAITING
+    assert a.state is RequestState.FINISHED and a.slot is None
+    if run_ahead:
+        assert b.state is RequestState.DECODE and b.num_computed == 3 and b.in_flight == 1
+    else:
+        assert b.state is RequestState.WAITING
     eng.step()
     assert b.state is RequestState.FINISHED and eng.cache.free_pages() == 1
     assert a.generated == plain_greedy(folder, [1, 4, 6], 1) and b.generated == plain_greedy(folder, [1, 5, 9], 1)
