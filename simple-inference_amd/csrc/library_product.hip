@@ -165,6 +165,23 @@ SIA_EXPORT int sia_blas_try_out(int on) {
     return 0;
 }
 
+// 0 if the library has an algorithm for the shape (found now, if the shape is new, and kept: nothing is launched or
+// timed), else as sia_blas_mm.  For callers that cannot take another way once they have begun.
+SIA_EXPORT int sia_blas_can(int M, int N, int K, int out_float) {
+    State* st = state_of_current_device();
+    if (!st) return 1;
+    if (M <= 0 || N <= 0 || K <= 0) return 2;
+    const uint64_t key = ((uint64_t)(uint32_t)M << 42) ^ ((uint64_t)(uint32_t)N << 21) ^ (uint64_t)(uint32_t)K ^
+                         ((uint64_t)(out_float ? 1 : 0) << 63);
+    auto it = st->plans.find(key);
+    if (it == st->plans.end()) {
+        Plan p;
+        make_plan(*st, p, M, N, K, out_float != 0, false, nullptr, nullptr, nullptr, nullptr);
+        it = st->plans.emplace(key, p).first;
+    }
+    return it->second.ok ? 0 : 3;
+}
+
 // 0: launched.  Anything else: nothing was launched (not initialised, or the library has no algorithm for the
 // shape), and the caller takes another way.
 SIA_EXPORT int sia_blas_mm(const void* X, const void* W, void* Y, int M, int N, int K, int out_float,

@@ -15,7 +15,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
-from typing import Optional
+from typing import Dict, Optional
 
 import torch
 
@@ -36,6 +36,7 @@ _SIGNATURES = {
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_attention_max_head_dim": [],
     "sia_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_prenorm_block": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "sia_sample": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "sia_sample_workspace_bytes": [_c_int],
     "sia_sample_static": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -108,6 +109,23 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
+class _BlockOwn(ctypes.Structure):
+    """``SiaBlockOwn`` of csrc/block.hip."""
+    _fields_ = ([(n, ctypes.c_void_p) for n in ("mixer_norm_gain", "w_qkv", "w_o", "feed_forward_norm_gain", "w_gate_up",
+                                               "w_down", "cos_table", "sin_table")]
+                + [(n, ctypes.c_float) for n in ("mixer_norm_eps", "feed_forward_norm_eps", "scale")]
+                + [(n, ctypes.c_int) for n in ("hidden", "n_heads", "n_kv", "head_dim", "rotary_dim", "inter", "window")])
+
+
+class _BlockStep(ctypes.Structure):
+    """``SiaBlockStep`` of csrc/block.hip."""
+    _fields_ = ([(n, ctypes.c_void_p) for n in ("product", "attend_single", "attend_runs", "residual", "normed", "qkv",
+                                               "attended", "mixed", "gate_up", "activated", "fed", "positions",
+                                               "seq_of_token", "cu_q", "kv_len", "ws_acc", "ws_ml")]
+                + [(n, ctypes.c_int) for n in ("n_tokens", "n_seqs", "n_single", "max_splits", "n_tiles", "n_tiles_split",
+                                               "n_tiles_long")])
+
+
 def _bind(lib, signatures):
     for name, argtypes in signatures.items():
         fn = getattr(lib, name)
@@ -135,6 +153,8 @@ class HipKernels:
         self.use_skinny_gemm = True      # few-row bfloat16 products by this package's kernel, not the library
         self.fuse_norms = True           # few rows: residual add in the product before a norm, row scale in the one after
         self.fuse_rope = True            # few rows: rotation and cache write in the q/k/v product
+        self.whole_blocks = True         # many rows: a block's launches in one call (``prenorm_block``)
+        self._products_known: Dict[tuple, bool] = {}
         self._skinny_rows = self.core.sia_gemm_skinny_max_rows()
         self.blas = self._load_blas()    # the BLAS library called directly; None: its products go through torch
 
@@ -148,6 +168,7 @@ class HipKernels:
             lib.sia_blas_mm.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
             lib.sia_blas_mm.restype = ctypes.c_int
             lib.sia_blas_try_out.argtypes, lib.sia_blas_try_out.restype = [_c_int], ctypes.c_int
+            lib.sia_blas_can.argtypes, lib.sia_blas_can.restype = [_c_int, _c_int, _c_int, _c_int], ctypes.c_int
             with torch.cuda.device(self.device):
                 if lib.sia_blas_init() != 0:
                     return None
@@ -567,6 +588,113 @@ class HipKernels:
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_tiles_split, n_tiles_long, n_heads,
                 n_kv_heads, cache.page_size, float(scale), window, self._stream()), "attn_prefill")
+
+    # -- a whole block in one call -------------------------------------------------
+    def _library_can(self, M, N, K) -> bool:
+        key = (M, N, K)
+        known = self._products_known.get(key)
+        if known is None:
+            with torch.cuda.device(self.device):
+                known = self._products_known[key] = self.blas.sia_blas_can(M, N, K, 0) == 0
+        return known
+
+    def _block_own(self, block):
+        """The block as the one-call form takes it (a structure of pointers and constants, with the tensors it points
+        into), or False if its parts are not of the kinds that form covers.  Made once and kept with the block."""
+        forms = block.plain_forms
+        if forms is not None:
+            return forms
+        block.plain_forms = False
+        parts = [getattr(p, "plain_form", lambda: None)()
+                 for p in (block.mixer_norm, block.mixer, block.feed_forward_norm, block.feed_forward)]
+        if any(f is None for f in parts) or [f["kind"] for f in parts] != ["rmsnorm", "paged_attention", "rmsnorm", "swiglu"]:
+            return False
+        n1, at, n2, ff = parts
+        H, nh, nkv, D, I = at["hidden"], at["n_heads"], at["n_kv_heads"], at["head_dim"], ff["inter"]
+        bf, f32 = torch.bfloat16, torch.float32
+        wanted = ((n1["weight"], f32, (H,)), (n2["weight"], f32, (H,)), (at["w_qkv"], bf, ((nh + 2 * nkv) * D, H)),
+                  (at["w_o"], bf, (H, nh * D)), (ff["w_gate_up"], bf, (2 * I, H)), (ff["w_down"], bf, (H, I)))
+        rd = at["rotary_dim"]
+        if rd:
+            wanted += ((at["cos"], f32, None), (at["sin"], f32, None))
+        for t, dtype, shape in wanted:
+            if (not isinstance(t, torch.Tensor) or t.device.type != "cuda" or t.dtype != dtype or not t.is_contiguous()
+                    or (shape is not None and tuple(t.shape) != shape)):
+                return False
+        if (ff["hidden"] != H or n1["size"] != H or n2["size"] != H or D % 16 or D > 256 or not at["scale"] > 0
+                or (rd and (at["cos"].shape[1] != rd // 2 or at["sin"].shape != at["cos"].shape))):
+            return False
+        own = _BlockOwn(_ptr(n1["weight"]), _ptr(at["w_qkv"]), _ptr(at["w_o"]), _ptr(n2["weight"]), _ptr(ff["w_gate_up"]),
+                        _ptr(ff["w_down"]), _ptr(at["cos"]) if rd else None, _ptr(at["sin"]) if rd else None,
+                        float(n1["eps"]), float(n2["eps"]), float(at["scale"]), H, nh, nkv, D, rd, I, int(at["window"] or 0))
+        block.plain_forms = (own, [t for t, _, _ in wanted], at["cos"].shape[0] if rd else None)
+        return block.plain_forms
+
+    def _block_step(self, own, ctx, device):
+        """What a step brings to the one-call form of its blocks of this geometry: buffers, metadata, the attention
+        plan.  Made once per step and geometry and kept with the step's context; None if the library has no
+        algorithm for one of the products at this number of rows."""
+        key = (own.hidden, own.n_heads, own.n_kv, own.head_dim, own.inter, own.window)
+        steps = getattr(ctx, "block_steps", None)
+        if steps is None:
+            try:
+                ctx.block_steps = steps = {}
+            except AttributeError:
+                return None
+        if key in steps:
+            return steps[key]
+        M, H, Q, I = ctx.n_tokens, own.hidden, own.n_heads * own.head_dim, own.inter
+        width = (own.n_heads + 2 * own.n_kv) * own.head_dim
+        steps[key] = None
+        if not all(self._library_can(M, n, k) for n, k in ((width, H), (H, Q), (2 * I, H), (H, I))):
+            return None
+        lib = self._attn_lib(own.head_dim)
+        n_dec, max_splits, ws_acc, ws_ml, tiles = self._attention_plan(lib, device, own.n_heads, own.n_kv, own.head_dim,
+                                                                       own.window, ctx)
+        new = lambda n: torch.empty((M, n), dtype=torch.bfloat16, device=device)
+        buffers = [new(H), new(width), new(Q), new(H), new(2 * I), new(I), new(H)]
+        fn = lambda f: ctypes.cast(f, ctypes.c_void_p).value
+        step = _BlockStep(fn(self.blas.sia_blas_mm), fn(lib.sia_attn_decode), fn(lib.sia_attn_prefill), None,
+                          *[_ptr(b) for b in buffers], _ptr(ctx.positions), _ptr(ctx.seq_of_token), _ptr(ctx.cu_q),
+                          _ptr(ctx.kv_len), _ptr(ws_acc), _ptr(ws_ml), M, ctx.n_seqs, n_dec, max_splits, *tiles)
+        steps[key] = (step, buffers)
+        return steps[key]
+
+    def prenorm_block(self, block, stream, ctx, cache) -> bool:
+        """Runs a pre-norm block of RMS norms, paged attention and SwiGLU on a step of many rows with one call into
+        the library (the same launches, in the same order, as the parts' own calls make); False, with nothing done,
+        where that form does not apply: the caller then goes part by part."""
+        if not self.whole_blocks or self.blas is None or not self.use_mfma_attention:
+            return False
+        residual = stream.residual
+        M = ctx.n_tokens
+        if (M <= self._skinny_rows or M > 65535 or getattr(ctx, "extra", None)
+                or residual.dtype != torch.float32 or cache.k_pages is None or cache.page_size < 8):
+            return False
+        made = self._block_own(block)
+        if not made:
+            return False
+        own, _, positions_covered = made
+        if (tuple(residual.shape) != (M, own.hidden) or not residual.is_contiguous() or cache.k_pages.dtype != torch.bfloat16
+                or (positions_covered is not None and positions_covered <= ctx.max_kv_len - 1)):
+            return False
+        step = self._block_step(own, ctx, residual.device)
+        if step is None:
+            return False
+        delta = stream.delta    # computes it if it is a product not yet computed
+        if delta is not None and (delta.dtype != torch.bfloat16 or tuple(delta.shape) != (M, own.hidden)
+                                  or not delta.is_contiguous()):
+            return False
+        self._check_pages(cache.k_pages, cache.v_pages, cache.block_table, cache.page_size, own.n_kv, own.head_dim,
+                          torch.bfloat16, ctx)
+        step_struct, buffers = step
+        step_struct.residual = _ptr(residual)
+        self._check(self.core.sia_prenorm_block(
+            ctypes.addressof(own), ctypes.addressof(step_struct), _ptr(delta), _ptr(cache.block_table),
+            cache.block_table.shape[1], _ptr(cache.k_pages), _ptr(cache.v_pages), cache.page_size, self._stream()),
+            "prenorm_block")
+        stream.delta = buffers[-1]
+        return True
 
     # -- sampling ------------------------------------------------------------------
     def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False, filters=None):

@@ -40,7 +40,7 @@ HIPCC_FLAGS = [
 # are specialisations compiled for the sizes a model has (see ``specialised``).
 LIBRARIES: Dict[str, Sequence[str]] = {
     "core": ("elementwise.hip", "rope_cache.hip", "attention_generic.hip", "gemm_generic.hip", "gemm_skinny.hip",
-             "sampling.hip", "bandwidth.hip"),
+             "sampling.hip", "bandwidth.hip", "block.hip"),
     # the vendor's BLAS library called directly (the products of steps of many tokens); optional: without it those
     # products go through torch
     "blas": ("library_product.hip",),

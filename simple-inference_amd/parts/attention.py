@@ -83,6 +83,17 @@ class Attention:
             self.w_qkv = tensors["q"].contiguous()
         self.w_o = tensors["o"].contiguous()
 
+    def plain_form(self):
+        """What this mixer is, as plain data, for kernels that can run a whole block in one call; None for the forms
+        that only ``forward`` covers (reading another layer's keys and values)."""
+        if not self.writes_kv:
+            return None
+        cos, sin = self.position.tables()
+        return {"kind": "paged_attention", "w_qkv": self.w_qkv, "w_o": self.w_o, "hidden": self.hidden,
+                "n_heads": self.num_heads, "n_kv_heads": self.num_kv_heads, "head_dim": self.head_dim,
+                "rotary_dim": self.position.rotary_dim, "cos": cos, "sin": sin, "scale": self.scale,
+                "window": self.window}
+
     def cache_need(self):
         return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
 

@@ -18,8 +18,14 @@ class PreNormBlock:
         self.feed_forward = feed_forward
         self.mixer_norm = mixer_norm
         self.feed_forward_norm = feed_forward_norm
+        self.plain_forms = None   # kept by kernels that run the block in one call: what they made of the parts
 
     def forward(self, stream, ctx, cache):
+        # Kernels that can make all of a block's launches in one call are shown the block (they look at what its
+        # parts say they are, ``plain_form``, and take it or leave it); else part by part.
+        whole = getattr(ctx.kernels, "prenorm_block", None)
+        if whole is not None and whole(self, stream, ctx, cache):
+            return
         h = _normed(self.mixer_norm, self.mixer, stream)
         stream.delta = self.mixer.forward(h, ctx, cache)
         h = _normed(self.feed_forward_norm, self.feed_forward, stream)

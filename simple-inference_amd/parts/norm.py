@@ -27,6 +27,10 @@ class RMSNorm:
 
     gives_scaled_rows = True
 
+    def plain_form(self):
+        """What this norm is, as plain data, for kernels that can run a whole block in one call."""
+        return {"kind": "rmsnorm", "weight": self.weight, "eps": self.eps, "size": self.size}
+
     def forward(self, stream, rows=None, scaled_ok=False):
         """Adds ``stream.delta`` into ``stream.residual`` and returns the normed rows.
 

@@ -38,6 +38,11 @@ class SwiGLU:
         self.w_gate_up = torch.cat([tensors["gate"], tensors["up"]], dim=0).contiguous()
         self.w_down = tensors["down"].contiguous()
 
+    def plain_form(self):
+        """What this feed-forward is, as plain data, for kernels that can run a whole block in one call."""
+        return {"kind": "swiglu", "w_gate_up": self.w_gate_up, "w_down": self.w_down, "hidden": self.hidden,
+                "inter": self.inter}
+
     def forward(self, h, ctx):
         k = self.env.kernels
         a = k.gated_linear(h, self.w_gate_up)   # the activation is fused into the product where a kernel has it

@@ -190,13 +190,13 @@ def test_float32_stored_weights_in_the_bfloat16_engine(tmp_path):
 def test_few_token_steps_take_the_products_with_fused_epilogues(folders):
     """Configuration D has the sizes for them: a step of few tokens in bfloat16 runs one product that rotates and
     writes the cache and two that add into the residual per layer, and no rotation or norm kernel between layers;
-    a step of many tokens runs none of them.  (That their logits agree with the plain implementation is what the
+    a step of many tokens runs none of them: its launches are made by one call a layer, or part by part.  (That their logits agree with the plain implementation is what the
     other tests of this file check, for D as for the others.)"""
     tiny = TINIES["d"]
     runner, cache, mcfg = make_runner(folders["d"], "hip-bf16", tiny.page_size, num_pages=64)
     core = runner.kernels.core
     counted = ("sia_gemm_skinny_rope", "sia_gemm_skinny_residual", "sia_gemm_skinny_swiglu", "sia_rope_kv_write",
-               "sia_add_rmsnorm")
+               "sia_add_rmsnorm", "sia_prenorm_block")
     calls = {name: 0 for name in counted}
     real = {name: getattr(core, name) for name in counted}
 
@@ -212,8 +212,15 @@ def test_few_token_steps_take_the_products_with_fused_epilogues(folders):
         layers = mcfg.num_hidden_layers
         tokens = random_tokens(mcfg.vocab_size, 40, seed=5)
         cache.admit("r")
-        runner.run([StepEntry("r", tokens[:37], [36])])       # many tokens: the library's products, separate kernels
-        assert calls["sia_gemm_skinny_rope"] == calls["sia_gemm_skinny_residual"] == 0
+        runner.run([StepEntry("r", tokens[:20], [19])])       # many tokens: the library's products, separate kernels,
+        assert calls["sia_gemm_skinny_rope"] == calls["sia_gemm_skinny_residual"] == 0    # launched by one call a layer
+        assert calls["sia_prenorm_block"] == layers and calls["sia_rope_kv_write"] == 0 and calls["sia_add_rmsnorm"] == 1
+        for name in counted:
+            calls[name] = 0
+        runner.kernels.whole_blocks = False                    # the same launches part by part
+        runner.run([StepEntry("r", tokens[20:37], [16])])
+        runner.kernels.whole_blocks = True
+        assert calls["sia_gemm_skinny_rope"] == calls["sia_gemm_skinny_residual"] == calls["sia_prenorm_block"] == 0
         assert calls["sia_rope_kv_write"] == layers and calls["sia_add_rmsnorm"] == 2 * layers + 1
         for name in counted:
             calls[name] = 0
