@@ -187,6 +187,36 @@ def test_float32_stored_weights_in_the_bfloat16_engine(tmp_path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", ["a", "d"])
+def test_a_block_in_one_call_is_the_block_part_by_part(folders, name):
+    """Steps of many tokens make a block's launches in one native call; the launches are the parts' own, so logits
+    and cache are the same bit for bit as part by part: prompt portions of changing size beside decoded tokens of
+    another request, whose pages are used again by a third."""
+    tiny = TINIES[name]
+    outs = []
+    for whole in (True, False):
+        runner, cache, mcfg = make_runner(folders[name], "hip-bf16", tiny.page_size, num_pages=-(-250 // tiny.page_size))
+        runner.kernels.whole_blocks = whole
+        a, b, c = (random_tokens(mcfg.vocab_size, n, seed=20 + i) for i, n in enumerate((150, 60, 90)))
+        schedule = [([(0, a[:70], [69]), (1, b[:30], [3, 29])], []),
+                    ([(1, [b[30]], [0]), (0, a[70:131], [0, 60])], []),
+                    ([(0, a[131:], [18]), (1, b[31:], list(range(29)))], [1]),
+                    ([(2, c[:64], [63]), (0, [a[-1]], [])], [0]),
+                    ([(2, c[64:], [25])], [2])]
+        got = replay(runner, cache, schedule)
+        outs.append((got, [g.k.clone() for g in cache.groups], [g.v.clone() for g in cache.groups]))
+        runner.kernels.whole_blocks = True
+    (got_whole, k_whole, v_whole), (got_parts, k_parts, v_parts) = outs
+    assert got_whole.keys() == got_parts.keys()
+    for req in got_whole:
+        assert got_whole[req].keys() == got_parts[req].keys()
+        for pos in got_whole[req]:
+            assert torch.equal(got_whole[req][pos], got_parts[req][pos]), (req, pos)
+    for x, y in zip(k_whole + v_whole, k_parts + v_parts):
+        assert torch.equal(x, y)
+
+
+@pytest.mark.gpu
 def test_few_token_steps_take_the_products_with_fused_epilogues(folders):
     """Configuration D has the sizes for them: a step of few tokens in bfloat16 runs one product that rotates and
     writes the cache and two that add into the residual per layer, and no rotation or norm kernel between layers;
