@@ -63,6 +63,26 @@ class PagePool:
         acct.pages.add(page)
         return page
 
+    def take_many(self, owner: int, n: int) -> List[int]:
+        """``take`` n times (a long prompt's first step takes a hundred pages and more): the same pages in the same
+        order; if there are not n for this owner, the error that the first missing one would have raised, and none
+        is taken."""
+        acct = self._account(owner)
+        against_promise = min(n, acct.promised)
+        if against_promise > self.n_free:
+            raise RuntimeError("a promised page is missing: more was promised than is free")
+        if n - against_promise > self.n_unpromised:
+            raise OutOfPages(f"owner {owner} holds no promise and every free page is promised to someone")
+        acct.promised -= against_promise
+        self._promised -= against_promise
+        held, returned, mine, taken = self._held, self._returned, acct.pages, []
+        for _ in range(n):
+            page = heapq.heappop(returned) if returned else self._next_fresh()
+            held[page] = 1
+            mine.add(page)
+            taken.append(page)
+        return taken
+
     def _next_fresh(self) -> int:
         self._fresh += 1
         return self._fresh - 1

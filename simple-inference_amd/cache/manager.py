@@ -94,8 +94,9 @@ class PagedGroup:
                     self.pool.drop(req, table[idx], restore_promise=True)
                     table[idx] = -1
                     self._touch(req)
-        while len(table) < pages_for(end, self.page_size):
-            table.append(self.pool.take(req))
+        more = pages_for(end, self.page_size) - len(table)
+        if more > 0:
+            table.extend(self.pool.take_many(req, more))
             self._touch(req)
 
     def _touch(self, req: int) -> None:

@@ -61,8 +61,10 @@ class StepRunner:
         used[0] = True
         return pinned.numpy()[:size], (pinned, copied)
 
-    def _check(self, entries: List[StepEntry]) -> None:
+    def _check(self, entries: List[StepEntry]) -> dict:
+        """Raises for entries that cannot run; returns every request's token ids as an array."""
         seen = set()
+        arrays = {}
         extra_keys = {key for e in entries if e.extra for key in e.extra}
         for e in entries:
             for key in extra_keys:
@@ -80,7 +82,7 @@ class StepRunner:
                 raise ValueError(
                     f"request {e.req} would reach position {self.cache.lengths[e.req] + len(e.tokens)}, "
                     f"beyond the engine's {self.max_positions}")
-            ids = np.asarray(e.tokens)      # checked as a whole: a prompt portion has thousands
+            ids = arrays[e.req] = np.asarray(e.tokens)      # checked as a whole: a prompt portion has thousands
             if ids.dtype.kind not in "iu":
                 raise ValueError(f"the token ids of request {e.req} are not integers ({ids.dtype})")
             if int(ids.min()) < 0 or int(ids.max()) >= self.vocab_size:
@@ -89,11 +91,12 @@ class StepRunner:
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"wanted place {w} of request {e.req} is outside its {len(e.tokens)} tokens")
+        return arrays
 
     def build_context(self, entries: List[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> StepContext:
         """Takes the pages the step needs and lays its metadata out on the device.  Entries with ``token_from``
         get their token id from ``device_tokens`` (int32, on the device), by a copy on the device."""
-        self._check(entries)
+        token_arrays = self._check(entries)
         from_device = [e for e in entries if e.token_from is not None]
         if from_device:
             if device_tokens is None or device_tokens.dtype != torch.int32:
@@ -127,7 +130,7 @@ class StepRunner:
         first_token = {}
         for s, e in enumerate(seqs):
             n = q_lens[s]
-            tok[t:t + n] = e.tokens
+            tok[t:t + n] = token_arrays[e.req]
             pos[t:t + n] = np.arange(starts[s], starts[s] + n, dtype=np.int32)
             sot[t:t + n] = s
             first_token[e.req] = t

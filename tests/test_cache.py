@@ -54,6 +54,36 @@ def test_pool_errors():
     a.audit()
 
 
+def test_many_pages_at_once_are_the_pages_one_by_one():
+    """``take_many`` hands out what as many calls of ``take`` would, against the promise first and then from the
+    unpromised pages, returned pages before fresh ones; if there are not enough, it takes none."""
+    rng = random.Random(3)
+    for _ in range(50):
+        pools = [PagePool(40), PagePool(40)]
+        promise, other = rng.randint(0, 12), rng.randint(0, 10)
+        for pool in pools:
+            pool.open(1, promise=promise)
+            pool.open(2, promise=other)
+            first = [pool.take(2) for _ in range(min(other, 6))]
+            for page in first[::2]:
+                pool.drop(2, page)      # returned pages, lower than the fresh ones, go out first
+        n = rng.randint(0, 45)
+        one_by_one, at_once = pools
+        try:
+            want = [one_by_one.take(1) for _ in range(n)]
+        except MemoryError:
+            want = None
+        if want is None:
+            before = (at_once.n_free, at_once.n_promised, at_once.pages(1))
+            with pytest.raises(MemoryError):
+                at_once.take_many(1, n)
+            assert (at_once.n_free, at_once.n_promised, at_once.pages(1)) == before
+        else:
+            assert at_once.take_many(1, n) == want
+            assert (at_once.n_free, at_once.n_promised) == (one_by_one.n_free, one_by_one.n_promised)
+        at_once.audit()
+
+
 def test_an_account_without_a_promise_takes_unpromised_pages_only():
     a = PagePool(3)
     a.open(1)
