@@ -130,6 +130,27 @@ def test_a_request_keeps_its_own_books():
     assert q.deliver(2, eos_ids=()) and q.finish_reason == "length"
     with pytest.raises(ValueError):
         req(3).take(1)                                       # not admitted
+    # an end by count is known before the last token is read: the request ends ahead and takes part in nothing more
+    e = req(2, max_new=2)
+    e.enter(1)
+    e.take(2), e.sampled(0)
+    assert not e.last_token_is_in_flight()
+    with pytest.raises(ValueError):
+        e.end_ahead()                                        # one more token may follow
+    assert e.deliver(5)
+    e.take(1), e.sampled(3)
+    assert e.last_token_is_in_flight()
+    e.end_ahead()
+    assert e.state is RequestState.ENDING and e.slot is None and e.tokens_wanted(8) == 0
+    assert e.deliver(7) and e.generated == [5, 7] and e.state is RequestState.FINISHED and e.finish_reason == "length"
+    s = Scheduler(max_running=2, token_budget=100, chunk_tokens=8)
+    a, b = req(3, max_new=1), req(3, max_new=4)
+    s.submit(a), s.submit(b)
+    assert ids(s.plan(lambda r: True)) == [(a.id, 3), (b.id, 3)]
+    for r in (a, b):
+        r.take(3), r.sampled(0)
+    a.end_ahead()
+    assert s.retire() == [a] and ids(s.plan()) == [(b.id, 1)]  # gone from the running before its token is read
 
 
 # ---- the engine on the CPU -----------------------------------------------------------------------
