@@ -81,6 +81,7 @@ def main(argv=None) -> int:
     else:
         engine = Engine.from_random(preset(args.random), args.seed, ecfg, generate_on_device=True)
     vocab = engine.model.vocab_size
+    print(engine.describe(), file=sys.stderr, flush=True)
 
     tokenizer = None
     if args.prompt is not None:

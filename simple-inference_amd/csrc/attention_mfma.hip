@@ -961,6 +961,13 @@ static DecodeMode decode_mode(int n_seqs, int n_heads, int n_kv, int max_splits)
     return DEC_PLAIN;
 }
 
+// Which of the three ways such a step takes (0 plain, 1 fold, 2 spread): for tests and profiles that want to know
+// which code ran.
+SIA_EXPORT int sia_attn_decode_mode(int n_seqs, int n_heads, int n_kv, int max_splits) {
+    if (n_seqs <= 0 || n_kv <= 0 || n_heads % n_kv || max_splits <= 0) return SIA_BAD_ARGUMENT;
+    return (int)decode_mode(n_seqs, n_heads, n_kv, max_splits);
+}
+
 // Floats of ws_acc and of ws_ml that sia_attn_decode needs for such a step (0: none, the pointer may be null).
 SIA_EXPORT long long sia_attn_decode_workspace(int n_seqs, int n_heads, int n_kv, int max_splits, int which) {
     if (n_seqs <= 0 || n_kv <= 0 || n_heads % n_kv || max_splits <= 0) return 0;

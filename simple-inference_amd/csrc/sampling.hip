@@ -573,6 +573,11 @@ static int scratch_address(SampleRow** out) {
 
 SIA_EXPORT int sia_sample_static_max_rows(void) { return SIA_SAMPLE_STATIC_MAX_ROWS; }
 
+SIA_EXPORT int sia_sample_static_init(void) {
+    SampleRow* ws = nullptr;
+    return scratch_address(&ws);
+}
+
 SIA_EXPORT int sia_sample_static(const float* logits, const float* temperature, const int* top_k, const float* top_p,
                                  const float* uniform, int* out, int rows, int vocab, int filters,
                                  hipStream_t stream) {

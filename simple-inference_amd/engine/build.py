@@ -36,10 +36,40 @@ def build_model(config_dict: Mapping, engine_cfg: EngineConfig, kernels):
     return DecoderModel(plan, env), model_cfg
 
 
+def count_parameters(model, model_cfg) -> int:
+    """Elements over all tensors the parts ask for (a shared tensor once).  Where the architecture's configuration
+    has a formula of its own for the count (reference: ``loader.py:301-316`` checks the total it loaded against
+    the known size of the model) the two must agree: the parts' shapes and the formula are written from the same
+    config.json keys by different code."""
+    total = 0
+    for spec in model.expected_tensors().values():
+        n = 1
+        for d in spec.shape:
+            n *= d
+        total += n
+    formula = getattr(model_cfg, "num_parameters", None)
+    if formula is not None and formula() != total:
+        raise ValueError(f"the model's parts hold {total:,} parameters, the configuration's formula says {formula():,}")
+    return total
+
+
+def describe(model, model_cfg, engine_cfg: EngineConfig) -> str:
+    """One line: architecture, parameters, bytes of the cache a token (reference: ``loader.py:301-316``,
+    ``config.py:144-149`` print the same two figures)."""
+    el = 2 if engine_cfg.dtype == "bfloat16" else 4
+    kv = sum(need.num_kv_heads * (need.head_dim + need.value_dim) * slabs * el
+             for need, slabs in zip(model.cache_layout().kv_groups, model.cache_layout().kv_slabs))
+    name = getattr(model_cfg, "architecture", type(model_cfg).__name__)
+    return (f"{name}: {count_parameters(model, model_cfg):,} parameters in {len(model.order)} layers, "
+            f"{kv:,} bytes of cache a token ({engine_cfg.dtype})")
+
+
 def model_from_folder(folder, engine_cfg: EngineConfig, kernels=None):
     kernels = kernels if kernels is not None else default_kernels()
     model, model_cfg = build_model(read_config_json(folder), engine_cfg, kernels)
-    tensors = load_weights(folder, model.expected_tensors(), engine_cfg.device, engine_cfg.torch_dtype)
+    count_parameters(model, model_cfg)
+    tensors = load_weights(folder, model.expected_tensors(), engine_cfg.device, engine_cfg.torch_dtype,
+                           duplicates=model.plan.duplicates)
     model.bind(tensors)
     return model, model_cfg
 

@@ -10,11 +10,13 @@ and one for decoded tokens (``serving/engine.py:330-349``).
 
 Running ahead: a decoding request's next input token is the sampler's output of the step before, which is on
 the device.  Who takes part in the next step, and with how many tokens, depends on the sampled tokens only through
-the ends of requests.  So when no request of the step on the GPU can reach ``max_new_tokens`` with the token it is
-about to get, the next step is planned and launched (admission included) before the host waits for those tokens,
-its token ids copied on the device; the GPU works while the host reads, books and plans.  ``step`` still reports one
-step's tokens per call, in order.  A request that turns out to have ended on an end-of-sequence token has then run
-one token too far; that token is dropped, and its slot goes to the next request a step later.
+the ends of requests.  So the next step is always planned and launched (admission included) before the host waits
+for the tokens of the step on the GPU, its token ids copied on the device; the GPU works while the host reads,
+books and plans.  The one end the host knows without reading a token is the end by count: a request whose token
+in flight is its last ends ahead (``ENDING``), takes part in no later step, and gives its pages and slot back
+before the next step is planned.  ``step`` still reports one step's tokens per call, in order.  A request that
+turns out to have ended on an end-of-sequence token has then run one token too far; that token is dropped, and its
+slot goes to the next request a step later.
 """
 
 from __future__ import annotations
@@ -73,6 +75,8 @@ class Engine:
         self._ahead = None   # a step launched but not yet read: (requests that sampled a token, those tokens)
         self._token_mirrors = None   # two pinned host buffers that sampled tokens are copied into, in turn
         self._mirror_turn = 0
+        self.model_folder = None   # where the model came from, if from a folder: a tokenizer file may lie beside it
+        self._tokenizer = None
         if engine_cfg.warmup:
             self.warmup()
 
@@ -82,7 +86,9 @@ class Engine:
         engine_cfg = engine_cfg or EngineConfig()
         kernels = kernels if kernels is not None else default_kernels()
         model, model_cfg = model_from_folder(folder, engine_cfg, kernels)
-        return cls(model, model_cfg, engine_cfg, kernels)
+        engine = cls(model, model_cfg, engine_cfg, kernels)
+        engine.model_folder = folder
+        return engine
 
     @classmethod
     def from_random(cls, config_dict, seed: int = 0, engine_cfg: Optional[EngineConfig] = None, kernels=None,
@@ -91,6 +97,11 @@ class Engine:
         kernels = kernels if kernels is not None else default_kernels()
         model, model_cfg = model_from_random(config_dict, seed, engine_cfg, kernels, **random_options)
         return cls(model, model_cfg, engine_cfg, kernels)
+
+    def describe(self) -> str:
+        """One line about the loaded model: parameters and cache bytes a token."""
+        from .build import describe
+        return describe(self.model, self.model_cfg, self.cfg)
 
     # -- requests ----------------------------------------------------------------
     def add_request(self, prompt_tokens: Sequence[int], max_new_tokens: Optional[int] = None,
@@ -311,10 +322,34 @@ class Engine:
         self.reset()
 
     # -- single-stream entry points ------------------------------------------------------
-    def generate(self, prompt_tokens: Sequence[int], max_new_tokens: int = 256, temperature: float = 1.0,
-                 top_k: int = 50, top_p: float = 0.9, seed: int = 0) -> Iterator[int]:
+    def tokenizer(self):
+        """The text front-end of the model folder (its ``tokenizer.json``); raises where there is none."""
+        if self._tokenizer is None:
+            if self.model_folder is None:
+                raise ValueError("this engine was not built from a model folder, so it has no tokenizer: give token ids")
+            from ..tokenizer import Tokenizer
+            self._tokenizer = Tokenizer.from_folder(self.model_folder, self.model.plan.bos_token_id)
+        return self._tokenizer
+
+    def generate(self, prompt, max_new_tokens: int = 256, temperature: float = 1.0,
+                 top_k: int = 50, top_p: float = 0.9, seed: int = 0) -> Iterator:
         """Yields the tokens of one request as they come; stops at EOS without yielding it
-        (reference: ``generate.py:50-119``, same option names and defaults)."""
+        (reference: ``generate.py:50-119``, same option names and defaults).  ``prompt`` is a list of token ids, and
+        token ids are yielded; or a text, as the reference takes it, if the model folder holds a ``tokenizer.json``:
+        then the pieces of text are yielded that each new token adds to the decoded output."""
+        if isinstance(prompt, str):
+            tok = self.tokenizer()
+            ids, shown = [], ""
+            for token in self.generate(tok.encode(prompt, add_bos=True), max_new_tokens, temperature, top_k, top_p,
+                                       seed):
+                ids.append(token)
+                text = tok.decode(ids)
+                if text.endswith("\ufffd"):     # half of a character that the next token completes
+                    continue
+                yield text[len(shown):]
+                shown = text
+            return
+        prompt_tokens = prompt
         req = self.add_request(prompt_tokens, params=SamplingParams(
             temperature=temperature, top_k=top_k, top_p=top_p, seed=seed, max_new_tokens=max_new_tokens))
         sent = 0
@@ -329,7 +364,13 @@ class Engine:
 
     def generate_with_stats(self, prompt_tokens: Sequence[int], max_new_tokens: int = 256, temperature: float = 1.0,
                             top_k: int = 50, top_p: float = 0.9, seed: int = 0, on_token=None):
-        """(tokens, stats) with the reference's stat names (``generate.py:227-237``)."""
+        """(tokens, stats) with the reference's stat names (``generate.py:227-237``); for a text prompt
+        (text, stats), as there."""
+        if isinstance(prompt_tokens, str):
+            tok = self.tokenizer()
+            tokens, stats = self.generate_with_stats(tok.encode(prompt_tokens, add_bos=True), max_new_tokens,
+                                                     temperature, top_k, top_p, seed, on_token)
+            return tok.decode(tokens), stats
         sync = (lambda: torch.cuda.synchronize(self.device)) if self.device.type == "cuda" else (lambda: None)
         if self.device.type == "cuda":
             torch.cuda.reset_peak_memory_stats(self.device)

@@ -137,7 +137,16 @@ class GraphedDecode:
             cu[:] = np.arange(size + 1)
             rows[:] = np.arange(size)
         n = len(entries)
-        starts = [cache.extend(e.req, 1) for e in entries]
+        starts = []
+        try:
+            for e in entries:
+                starts.append(cache.extend(e.req, 1))
+        except Exception:
+            # a request that found no page (replay without promises): the ones before it give theirs back, so
+            # that the books are as they were before the call
+            for e in entries[:len(starts)]:
+                cache.retract(e.req, 1)
+            raise
         tok[:n] = [e.tokens[0] for e in entries]
         pos[:n] = starts
         kvl[:n] = pos[:n] + 1

@@ -41,6 +41,7 @@ _SIGNATURES = {
     "sia_sample_workspace_bytes": [_c_int],
     "sia_sample_static": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "sia_sample_static_max_rows": [],
+    "sia_sample_static_init": [],
     "sia_gemm_skinny": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_gemm_skinny_max_rows": [],
     "sia_gemm_skinny_residual_blocks": [_c_int],
@@ -61,6 +62,7 @@ _ATTN_SIGNATURES = {
                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "sia_attn_decode_max_splits": [_c_int, _c_int],
     "sia_attn_decode_workspace": [_c_int, _c_int, _c_int, _c_int, _c_int],
+    "sia_attn_decode_mode": [_c_int, _c_int, _c_int, _c_int],
     "sia_attn_prefill_rows": [],
     "sia_attn_prefill_rows_split": [],
     "sia_attn_prefill_rows_long": [],

@@ -55,6 +55,8 @@ def llama_plan(cfg: LlamaConfig) -> ModelPlan:
         bos_token_id=cfg.bos_token_id,
         eos_token_ids=cfg.eos_token_ids,
         max_position_embeddings=cfg.max_position_embeddings,
+        # a tied model whose file also stores the head (reference: ``model/llama.py:147-154`` reads it if present)
+        duplicates={"lm_head.weight": "model.embed_tokens.weight"} if cfg.tie_word_embeddings else {},
     )
 
 

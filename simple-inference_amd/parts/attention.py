@@ -86,8 +86,8 @@ class Attention:
     def plain_form(self):
         """What this mixer is, as plain data, for kernels that can run a whole block in one call; None for the forms
         that only ``forward`` covers (reading another layer's keys and values)."""
-        if not self.writes_kv:
-            return None
+        if not self.writes_kv or type(self).forward is not Attention.forward:
+            return None     # a subclass with a forward of its own is no longer what this form describes
         cos, sin = self.position.tables()
         return {"kind": "paged_attention", "w_qkv": self.w_qkv, "w_o": self.w_o, "hidden": self.hidden,
                 "n_heads": self.num_heads, "n_kv_heads": self.num_kv_heads, "head_dim": self.head_dim,

@@ -35,18 +35,22 @@ class CacheLayout:
     run_state: List[Optional[int]] = field(default_factory=list)
 
 
+_REGISTRY_OF_ROLE = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}
+
+
 class _Layer:
+    """The parts a ``LayerSpec`` names, built, and the block that arranges them.  The block kind is given the parts
+    as keyword arguments under the spec's names and says by its constructor which it takes."""
+
     def __init__(self, spec, env):
-        self.mixer = MIXERS.get(spec.mixer.kind)(spec.mixer.params, env)
-        self.feed_forward = FEED_FORWARDS.get(spec.feed_forward.kind)(spec.feed_forward.params, env)
-        self.mixer_norm = NORMS.get(spec.mixer_norm.kind)(spec.mixer_norm.params, env)
-        self.feed_forward_norm = NORMS.get(spec.feed_forward_norm.kind)(spec.feed_forward_norm.params, env)
-        self.block = BLOCKS.get(spec.block)(
-            self.mixer, self.feed_forward, self.mixer_norm, self.feed_forward_norm)
-        self.parts = [
-            (self.mixer, spec.mixer), (self.feed_forward, spec.feed_forward),
-            (self.mixer_norm, spec.mixer_norm), (self.feed_forward_norm, spec.feed_forward_norm),
-        ]
+        self.named = {name: _REGISTRY_OF_ROLE[ps.role].get(ps.kind)(ps.params, env) for name, ps in spec.parts.items()}
+        block_cls = BLOCKS.get(spec.block)
+        try:
+            self.block = block_cls(**self.named)
+        except TypeError as exc:
+            raise ValueError(f"a {spec.block!r} block does not take the parts {sorted(self.named)}: {exc}") from None
+        self.mixer = next((self.named[name] for name, ps in spec.parts.items() if ps.role == "mixer"), None)
+        self.parts = [(self.named[name], ps) for name, ps in spec.parts.items()]
 
 
 class DecoderModel:
@@ -88,14 +92,17 @@ class DecoderModel:
         """Hands every part its tensors (already checked, placed and typed by the loader)."""
         for part, spec in self._parts:
             part.bind({local: tensors[spec.weights[local]] for local in part.weight_specs()})
+        for layer in self.layers:
+            if getattr(layer.block, "plain_forms", None) is not None:
+                layer.block.plain_forms = None     # what kernels kept of the parts pointed into the old tensors
 
     # -- caches ------------------------------------------------------------
     def _make_cache_layout(self) -> CacheLayout:
         layout = CacheLayout()
         latest_run_of_layer: Dict[int, int] = {}
         for e, li in enumerate(self.order):
-            mixer = self.layers[li].mixer
-            need = mixer.cache_need()
+            mixer = self.layers[li].mixer       # None: a layer without a mixer owns neither pages nor state
+            need = mixer.cache_need() if mixer is not None else None
             source = getattr(mixer, "kv_from_layer", None)
             if need is None:
                 layout.run_kv.append(None)
@@ -113,7 +120,7 @@ class DecoderModel:
                 g = layout.kv_groups.index(need)
                 layout.run_kv.append((g, layout.kv_slabs[g]))
                 layout.kv_slabs[g] += 1
-            sneed = mixer.state_need()
+            sneed = mixer.state_need() if mixer is not None else None
             if sneed is None:
                 layout.run_state.append(None)
             else:

@@ -28,7 +28,10 @@ class RMSNorm:
     gives_scaled_rows = True
 
     def plain_form(self):
-        """What this norm is, as plain data, for kernels that can run a whole block in one call."""
+        """What this norm is, as plain data, for kernels that can run a whole block in one call (None for a
+        subclass with a forward of its own: it is no longer what this form describes)."""
+        if type(self).forward is not RMSNorm.forward:
+            return None
         return {"kind": "rmsnorm", "weight": self.weight, "eps": self.eps, "size": self.size}
 
     def forward(self, stream, rows=None, scaled_ok=False):

@@ -17,8 +17,9 @@ Interfaces (``env`` is a ``BuildEnv``; ``ctx`` a ``StepContext``):
   delta into its 32-bit residual and returns the normalised rows.
 * position encoding: whatever its mixer consumes; the rotary kind gives
   ``tables(device) -> (cos, sin)`` indexed by absolute position.
-* block: ``__init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm)``,
-  ``forward(stream, ctx, cache) -> None``.
+* block: ``__init__(self, **parts)`` with the names it gives its parts as keyword arguments (the pre-norm
+  block: ``mixer, feed_forward, mixer_norm, feed_forward_norm``; a ``LayerSpec`` names the parts of its
+  layer under those names), ``forward(stream, ctx, cache) -> None``.
 * embedding: ``forward(ctx) -> Tensor[N, hidden]`` float32, the residual stream's start.
 * head: ``forward(h) -> Tensor[rows, vocab]`` float32 logits; a head that can use the embedding's
   matrix has ``share_embedding(embedding)``, called before ``bind`` when its params say ``tied``.

@@ -39,7 +39,10 @@ class SwiGLU:
         self.w_down = tensors["down"].contiguous()
 
     def plain_form(self):
-        """What this feed-forward is, as plain data, for kernels that can run a whole block in one call."""
+        """What this feed-forward is, as plain data, for kernels that can run a whole block in one call (None for
+        a subclass with a forward of its own: it is no longer what this form describes)."""
+        if type(self).forward is not SwiGLU.forward:
+            return None
         return {"kind": "swiglu", "w_gate_up": self.w_gate_up, "w_down": self.w_down, "hidden": self.hidden,
                 "inter": self.inter}
 

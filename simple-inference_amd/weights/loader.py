@@ -27,10 +27,11 @@ from ..parts.plan import TensorSpec
 class WeightError(ValueError):
     """The checkpoint does not hold what the model wants; lists all differences."""
 
-    def __init__(self, missing, unexpected, wrong_shape, where=""):
+    def __init__(self, missing, unexpected, wrong_shape, where="", differing=()):
         self.missing = list(missing)
         self.unexpected = list(unexpected)
         self.wrong_shape = list(wrong_shape)
+        self.differing = list(differing)   # (name, the tensor it should repeat): stored twice with different values
         lines = [f"checkpoint {where} does not match the model:".replace("  ", " ")]
         if self.missing:
             lines.append(f"  missing ({len(self.missing)}): " + ", ".join(self.missing))
@@ -39,6 +40,9 @@ class WeightError(ValueError):
         if self.wrong_shape:
             lines.append(f"  wrong shape ({len(self.wrong_shape)}): " + ", ".join(
                 f"{n} is {list(got)}, wanted {list(want)}" for n, got, want in self.wrong_shape))
+        if self.differing:
+            lines.append(f"  stored twice with different values ({len(self.differing)}): " + ", ".join(
+                f"{n} is not equal to {other}, which the configuration says it shares" for n, other in self.differing))
         super().__init__("\n".join(lines))
 
 
@@ -75,19 +79,29 @@ def target_dtype(stored: torch.dtype, role: str, compute: torch.dtype) -> torch.
 
 
 def check_names_and_shapes(found: Mapping[str, Tuple[int, ...]], expected: Mapping[str, TensorSpec],
-                           ignore_suffixes: Iterable[str] = (), where: str = "") -> None:
+                           ignore_suffixes: Iterable[str] = (), where: str = "",
+                           duplicates: Mapping[str, str] = {}) -> None:
     ignore = tuple(ignore_suffixes)
     missing = [n for n in expected if n not in found]
-    unexpected = [n for n in found if n not in expected and not (ignore and n.endswith(ignore))]
+    unexpected = [n for n in found if n not in expected and n not in duplicates and not (ignore and n.endswith(ignore))]
     wrong = [(n, tuple(found[n]), tuple(expected[n].shape)) for n in expected
              if n in found and tuple(found[n]) != tuple(expected[n].shape)]
+    wrong += [(n, tuple(found[n]), tuple(expected[other].shape)) for n, other in duplicates.items()
+              if n in found and n not in expected and other in expected
+              and tuple(found[n]) != tuple(expected[other].shape)]
     if missing or unexpected or wrong:
         raise WeightError(sorted(missing), sorted(unexpected), wrong, where)
 
 
 def load_weights(folder, expected: Mapping[str, TensorSpec], device, compute_dtype: torch.dtype,
-                 ignore_suffixes: Iterable[str] = ("rotary_emb.inv_freq",)) -> Dict[str, torch.Tensor]:
-    """Reads the tensors named in ``expected`` from a model folder onto ``device``."""
+                 ignore_suffixes: Iterable[str] = ("rotary_emb.inv_freq",),
+                 duplicates: Mapping[str, str] = {}) -> Dict[str, torch.Tensor]:
+    """Reads the tensors named in ``expected`` from a model folder onto ``device``.
+
+    ``duplicates`` maps names a checkpoint may hold beside the expected ones to the expected tensor each must
+    repeat (a tied model stored with its ``lm_head.weight``: the reference takes such a file,
+    ``model/llama.py:147-154``).  A duplicate equal to its tensor is passed over; one that differs is an error,
+    since the engine would compute with one of the two and the file means the other."""
     from safetensors import safe_open
 
     folder = Path(folder)
@@ -97,7 +111,12 @@ def load_weights(folder, expected: Mapping[str, TensorSpec], device, compute_dty
         for path in set(shards.values()):
             handles[path] = safe_open(str(path), framework="pt")
         shapes = {name: tuple(handles[path].get_slice(name).get_shape()) for name, path in shards.items()}
-        check_names_and_shapes(shapes, expected, ignore_suffixes, where=str(folder))
+        duplicates = {n: other for n, other in duplicates.items() if n not in expected and other in expected}
+        check_names_and_shapes(shapes, expected, ignore_suffixes, where=str(folder), duplicates=duplicates)
+        differing = [(n, other) for n, other in sorted(duplicates.items()) if n in shards and not torch.equal(
+            handles[shards[n]].get_tensor(n).float(), handles[shards[other]].get_tensor(other).float())]
+        if differing:
+            raise WeightError((), (), (), str(folder), differing)
         out: Dict[str, torch.Tensor] = {}
         for name, spec in expected.items():
             t = handles[shards[name]].get_tensor(name)

@@ -24,13 +24,17 @@ import torch
 # configuration and weights
 # ---------------------------------------------------------------------------
 
+def read_config(folder):
+    with open(Path(folder) / "config.json") as f:
+        return json.load(f)
+
+
 def read_model(folder, dtype=torch.float32):
     """(config dict, {tensor name: tensor}) of a model folder."""
     from safetensors.torch import load_file
 
     folder = Path(folder)
-    with open(folder / "config.json") as f:
-        cfg = json.load(f)
+    cfg = read_config(folder)
     tensors = {k: v.to(dtype) for k, v in load_file(str(folder / "model.safetensors")).items()}
     return cfg, tensors
 
@@ -99,14 +103,16 @@ def apply_rope(x, cos, sin):
     return x * cos[:, None, :] + rotate_half(x) * sin[:, None, :]
 
 
-def attention(q, k, v, q_positions, k_positions, scale=None, window=None):
+def attention(q, k, v, q_positions, k_positions, scale=None, window=None, rnd=None):
     """Scores, mask, softmax, weighted sum.
 
     q [Tq, Hq, D]; k, v [Tk, Hkv, D].  reference: kernels/attention_kernel.py:184-251 —
     query head h reads kv head h // (Hq // Hkv); S = (q . k) * scale with
     scale = 1 / sqrt(D) applied after the dot; key j visible iff position(j) <= position(query)
     (serving/paged_kv_cache.py:366-375 writes the same mask explicitly); softmax over the
-    visible keys; O = P V.  ``window`` w additionally hides keys at distance >= w.
+    visible keys; O = P V.  ``window`` w additionally hides keys at distance >= w.  ``rnd`` (see
+    ``forward_as_the_reference_rounds``) is applied to the probabilities before P V
+    (kernels/attention_kernel.py:241 casts p to the values' dtype).
     """
     Tq, Hq, D = q.shape
     Tk, Hkv, _ = k.shape
@@ -123,6 +129,10 @@ def attention(q, k, v, q_positions, k_positions, scale=None, window=None):
         scores = (q[:, h, :] @ kh.T) * scale
         scores = scores.masked_fill(~visible, float("-inf"))
         probs = torch.softmax(scores, dim=-1)
+        if rnd is not None:
+            # the kernel rounds exp(s - m) before P V and divides the float sum at the end; rounding the
+            # normalised probabilities instead differs by the rounding of one common factor
+            probs = rnd(probs)
         out[:, h, :] = probs @ vh
     return out
 
@@ -163,15 +173,74 @@ def forward(cfg, w, tokens, start_position=0, rows=None):
     """Logits [T, V] of one whole sequence (with ``rows``: at those places only, [len(rows), V]; the layers
     still see the whole sequence).  reference: model/llama.py:173-186 —
     embed -> blocks -> norm -> head; tied head = embedding matrix (ops/embedding.py:84-92)."""
-    tokens = torch.as_tensor(tokens, dtype=torch.long)
-    positions = torch.arange(start_position, start_position + len(tokens))
-    inv_freq = rope_inv_freq(head_dim_of(cfg), float(cfg["rope_theta"]), cfg.get("rope_scaling"))
+    device = w["model.embed_tokens.weight"].device      # the weights may lie on a GPU: then so does everything
+    tokens = torch.as_tensor(tokens, dtype=torch.long, device=device)
+    positions = torch.arange(start_position, start_position + len(tokens), device=device)
+    inv_freq = rope_inv_freq(head_dim_of(cfg), float(cfg["rope_theta"]), cfg.get("rope_scaling")).to(device)
     x = w["model.embed_tokens.weight"][tokens]
     for i in range(cfg["num_hidden_layers"]):
         x = block(x, positions, w, i, cfg, inv_freq)
     if rows is not None:
-        x = x[torch.as_tensor(rows, dtype=torch.long)]
+        x = x[torch.as_tensor(rows, dtype=torch.long, device=device)]
     x = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
+    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", True) else w["lm_head.weight"]
+    return x @ head.T
+
+
+# ---------------------------------------------------------------------------
+# the same model with the reference's bfloat16 roundings
+# ---------------------------------------------------------------------------
+
+def to_bfloat16_and_back(t):
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
+def forward_as_the_reference_rounds(cfg, w, tokens, rows=None, rnd=to_bfloat16_and_back):
+    """``forward`` with every intermediate result rounded where the reference's bfloat16 model materialises a
+    bfloat16 tensor on its production path (the fused kernels: one rounding each).  Computed in the weights' dtype
+    (float64 for a yardstick) apart from those roundings, it shows how far a *correct* bfloat16 implementation of
+    this model lies from exact arithmetic on given weights and tokens: the measure for what a bfloat16 engine may
+    differ by.  Places, in the order of a block (model/block.py:135-147):
+
+    * the norm's output (kernels/rmsnorm_kernel.py:105-113: float statistics and gain, one rounding);
+    * q, k, v as the products leave the BLAS library (ops/attention.py:128-130);
+    * the cos/sin rows, cast to the activations' dtype (ops/attention.py:143-145), and the rotated q and k
+      (kernels/rope_kernel.py:131-154: float arithmetic, one rounding);
+    * the probabilities before P V (kernels/attention_kernel.py:241) and the attention's output (:250);
+    * the output projection (ops/attention.py:226) and the residual sum, which the reference keeps in the
+      activations' dtype (model/block.py:139);
+    * gate and up (ops/mlp.py:117), silu(gate) * up (kernels/swiglu_kernel.py:142-150: float, one rounding),
+      the down projection (ops/mlp.py:128) and the second residual sum (model/block.py:145);
+    * the last norm (model/llama.py:181).  The logits are left as the exact product of that rounded row: the
+      reference rounds them too (model/llama.py:184), which a bound should not profit from.
+    """
+    device = w["model.embed_tokens.weight"].device
+    tokens = torch.as_tensor(tokens, dtype=torch.long, device=device)
+    T = len(tokens)
+    positions = torch.arange(T, device=device)
+    Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], head_dim_of(cfg)
+    eps = cfg["rms_norm_eps"]
+    inv_freq = rope_inv_freq(D, float(cfg["rope_theta"]), cfg.get("rope_scaling")).to(device)
+    x = w["model.embed_tokens.weight"][tokens]
+    cos, sin = rope_tables(positions, inv_freq, x.dtype)
+    cos, sin = rnd(cos), rnd(sin)
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}"
+        h = rnd(rms_norm(x, w[f"{p}.input_layernorm.weight"], eps))
+        q = rnd(h @ w[f"{p}.self_attn.q_proj.weight"].T).view(T, Hq, D)
+        k = rnd(h @ w[f"{p}.self_attn.k_proj.weight"].T).view(T, Hkv, D)
+        v = rnd(h @ w[f"{p}.self_attn.v_proj.weight"].T).view(T, Hkv, D)
+        q, k = rnd(apply_rope(q, cos, sin)), rnd(apply_rope(k, cos, sin))
+        o = rnd(attention(q, k, v, positions, positions, rnd=rnd))
+        x = rnd(x + rnd(o.reshape(T, Hq * D) @ w[f"{p}.self_attn.o_proj.weight"].T))
+        h = rnd(rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], eps))
+        g = rnd(h @ w[f"{p}.mlp.gate_proj.weight"].T)
+        u = rnd(h @ w[f"{p}.mlp.up_proj.weight"].T)
+        a = rnd((g * torch.sigmoid(g)) * u)
+        x = rnd(x + rnd(a @ w[f"{p}.mlp.down_proj.weight"].T))
+    if rows is not None:
+        x = x[torch.as_tensor(rows, dtype=torch.long, device=device)]
+    x = rnd(rms_norm(x, w["model.norm.weight"], eps))
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", True) else w["lm_head.weight"]
     return x @ head.T
 

@@ -1,6 +1,5 @@
 """What the measurement program promises without a GPU: its options, and its refusal of more than one GPU."""
 
-import json
 import os
 import subprocess
 import sys
@@ -37,7 +36,6 @@ def test_flops_and_bytes_of_the_headline_shape():
     layers, head = bench.matmul_params(mc)
     assert layers == 28 * 100_663_296 and head == 128256 * 3072
     assert mc.kv_bytes_per_token(2) == 28 * 8 * 128 * 2 * 2
-    json.dumps({"ok": True})
 
 
 def test_decode_allowance_covers_the_steps_that_build_the_contexts():

@@ -734,3 +734,140 @@ def test_a_second_position_axis_reaches_a_part_through_the_step(tmp_path):
     finally:
         unregister_architecture("ToyTwoAxis")
         MIXERS.unregister("test_two_axis")
+
+
+# ---- blocks of other kinds: a third norm, no feed-forward, no mixer -------------------------------------------------
+class SandwichBlock:
+    """x += post_norm(mixer(norm1(x))); x += feed_forward(norm2(x)): a block with three norms, of which one
+    normalises a part's output before it is added.  It takes its parts under names of its own choosing."""
+
+    def __init__(self, mixer, feed_forward, mixer_norm, after_mixer_norm, feed_forward_norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.after_mixer_norm, self.feed_forward_norm = mixer_norm, after_mixer_norm, feed_forward_norm
+
+    def forward(self, stream, ctx, cache):
+        from simple_inference_amd.parts.context import ResidualStream
+        h = self.mixer_norm.forward(stream)
+        mixed = self.mixer.forward(h, ctx, cache)
+        mixed = mixed.compute() if hasattr(mixed, "compute") else mixed
+        # the norm of the output: a stream of its own whose residual is the output itself
+        stream.delta = self.after_mixer_norm.forward(ResidualStream(mixed.float()))
+        h = self.feed_forward_norm.forward(stream)
+        stream.delta = self.feed_forward.forward(h, ctx)
+
+
+class MixerOnlyBlock:
+    """x += mixer(norm(x)), and nothing else."""
+
+    def __init__(self, mixer, norm):
+        self.mixer, self.norm = mixer, norm
+
+    def forward(self, stream, ctx, cache):
+        stream.delta = self.mixer.forward(self.norm.forward(stream), ctx, cache)
+
+
+class FeedForwardOnlyBlock:
+    """x += feed_forward(norm(x)): a layer without a mixer owns no pages and no state."""
+
+    def __init__(self, feed_forward, norm):
+        self.feed_forward, self.norm = feed_forward, norm
+
+    def forward(self, stream, ctx, cache):
+        assert cache.k_pages is None and cache.state is None
+        stream.delta = self.feed_forward.forward(self.norm.forward(stream), ctx)
+
+
+def other_blocks_plan(cfg):
+    P = PartSpec
+    norm = lambda name: P("rmsnorm", {"size": H, "eps": 1e-5}, {"weight": name}, role="norm")
+    rope = {"kind": "rope", "params": {"rotary_dim": 16, "theta": 10000.0, "scaling": None}}
+    attn = lambda p: P("attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 2, "head_dim": 16, "position": rope},
+                       {k: f"{p}.{k}" for k in "qkvo"}, role="mixer")
+    ffn = lambda p: P("swiglu", {"hidden_size": H, "intermediate_size": 48},
+                      {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"}, role="feed_forward")
+    layers = [
+        LayerSpec(block="test_sandwich", mixer=attn("l0.attn"), feed_forward=ffn("l0.ffn"), mixer_norm=norm("l0.n1"),
+                  feed_forward_norm=norm("l0.n2"), parts={"after_mixer_norm": norm("l0.n3")}),
+        LayerSpec(block="test_mixer_only", parts={"mixer": attn("l1.attn"), "norm": norm("l1.n")}),
+        LayerSpec(block="test_feed_forward_only", parts={"feed_forward": ffn("l2.ffn"), "norm": norm("l2.n")}),
+    ]
+    return ModelPlan(hidden_size=H, vocab_size=V,
+                     embedding=P("embedding", {"vocab_size": V, "hidden_size": H}, {"weight": "embed"}),
+                     layers=layers, order=[0, 2, 1, 2], final_norm=norm("final"),
+                     head=P("head", {"vocab_size": V, "hidden_size": H, "tied": True}, {}))
+
+
+def other_blocks_reference(w, tokens):
+    import plain_llama as plain
+    w = {k: v.double() for k, v in w.items()}
+    T = len(tokens)
+    pos = torch.arange(T)
+    cos, sin = plain.rope_tables(pos, plain.rope_inv_freq(16, 10000.0), torch.float64)
+    norm = lambda x, name: plain.rms_norm(x, w[name], 1e-5)
+
+    def attend(h, p):
+        q = plain.apply_rope((h @ w[f"{p}.q"].T).view(T, 2, 16), cos, sin)
+        k = plain.apply_rope((h @ w[f"{p}.k"].T).view(T, 2, 16), cos, sin)
+        v = (h @ w[f"{p}.v"].T).view(T, 2, 16)
+        return plain.attention(q, k, v, pos, pos).reshape(T, 32) @ w[f"{p}.o"].T
+
+    ffn = lambda h, p: plain.swiglu_mlp(h, w[f"{p}.gate"], w[f"{p}.up"], w[f"{p}.down"])
+    x = w["embed"][tokens]
+    x = x + norm(attend(norm(x, "l0.n1"), "l0.attn"), "l0.n3")
+    x = x + ffn(norm(x, "l0.n2"), "l0.ffn")
+    x = x + ffn(norm(x, "l2.n"), "l2.ffn")
+    x = x + attend(norm(x, "l1.n"), "l1.attn")
+    x = x + ffn(norm(x, "l2.n"), "l2.ffn")
+    return norm(x, "final") @ w["embed"].T
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_blocks_with_a_third_norm_without_a_feed_forward_and_without_a_mixer(backend):
+    """A layer is a block kind and the named parts that kind arranges: three block kinds defined here take parts
+    under names of their own (a third norm; a mixer and one norm; a feed-forward and one norm), are registered
+    from outside and run beside one another in one model.  The layer without a mixer owns no pages."""
+    from simple_inference_amd.parts import BLOCKS, register_block
+    for kind, cls in (("test_sandwich", SandwichBlock), ("test_mixer_only", MixerOnlyBlock),
+                      ("test_feed_forward_only", FeedForwardOnlyBlock)):
+        register_block(kind, cls, replace=True)
+    register_architecture("ToyOtherBlocks", lambda d: d, other_blocks_plan, replace=True)
+    try:
+        runner, cache, weights = make(backend, {"architectures": ["ToyOtherBlocks"]})
+        layout = runner.model.cache_layout()
+        assert layout.run_kv == [(0, 0), None, (0, 1), None] and layout.kv_slabs == [2] and not layout.states
+        tokens = torch.randint(0, V, (21,), generator=torch.Generator().manual_seed(8)).tolist()
+        ref = other_blocks_reference(weights, tokens)
+        cache.admit(1)
+        got, fed = [], 0
+        for n in (8, 1, 2, 1, 6, 3):
+            got.append(runner.run([StepEntry(1, tokens[fed:fed + n], list(range(n)))]))
+            fed += n
+        assert rel_err(torch.cat(got), ref) < (2.5e-2 if backend == "hip-bf16" else 3e-5)
+        cache.release(1)
+        cache.check()
+        # a block kind is told by name which parts it does not take
+        register_architecture("ToyWrongParts", lambda d: d, lambda cfg: ModelPlan(
+            hidden_size=H, vocab_size=V, embedding=other_blocks_plan(cfg).embedding,
+            layers=[LayerSpec(block="test_mixer_only", mixer=other_blocks_plan(cfg).layers[1].parts["mixer"])],
+            final_norm=other_blocks_plan(cfg).final_norm, head=other_blocks_plan(cfg).head), replace=True)
+        with pytest.raises(ValueError, match="test_mixer_only.*does not take the parts"):
+            make(backend, {"architectures": ["ToyWrongParts"]})
+    finally:
+        unregister_architecture("ToyOtherBlocks")
+        unregister_architecture("ToyWrongParts")
+        for kind in ("test_sandwich", "test_mixer_only", "test_feed_forward_only"):
+            BLOCKS.unregister(kind)
+
+
+def test_a_layer_spec_says_what_is_wrong_with_its_parts():
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5}, {"weight": "n"})
+    with pytest.raises(ValueError, match="role"):
+        LayerSpec(block="x", parts={"some_norm": norm})                       # a free name needs a role
+    mixer = PartSpec("attention", {}, {}, role="mixer")
+    with pytest.raises(ValueError, match="at most one"):
+        LayerSpec(block="x", mixer=mixer, parts={"second": PartSpec("attention", {}, {}, role="mixer")})
+    with pytest.raises(ValueError, match="twice"):
+        LayerSpec(block="x", mixer=mixer, parts={"mixer": mixer})
+    spec = LayerSpec(mixer=mixer, parts={"mixer_norm": norm})                # the four known names carry their roles
+    assert spec.parts["mixer_norm"].role == "norm" and spec.mixer_norm is spec.parts["mixer_norm"]
+    assert list(spec.parts) == ["mixer_norm", "mixer"]

@@ -575,7 +575,8 @@ def test_matrix_core_attention_runs_longer_than_a_block_table_window(hip, monkey
 def test_attention_finds_one_key_at_every_kind_of_edge(hip, dtype, q_len):
     """One key among hundreds is made to stand out; the output must be its value row.  The key is put at
     the edges where an indexing fault would lose it: first and last offset of a page, of a 32- and
-    64-key tile, of a 256-key split, the first key, the newest key, and both sides of a window's edge."""
+    64-key tile, the first key, the newest key, and both sides of a window's edge.  (700 keys are 22 tiles, which
+    the decode kernel does not split; longer sequences and their splits have a test of their own below.)"""
     n_heads, n_kv, D, ps = 4, 2, 64, 16
     kv = 700
     ctx = Ctx([q_len], [kv])
@@ -603,6 +604,73 @@ def test_attention_finds_one_key_at_every_kind_of_edge(hip, dtype, q_len):
             want = cache.v_pages[page, h // 2, :, far % ps].float()
             close = torch.allclose(row[h], want, rtol=2e-2, atol=2e-2)
             assert close == seen, (far, win, h)
+
+
+def _decode_splits(n_tiles):
+    """How many workgroups share a sequence of that many visible key tiles (the kernel's own rule, written down a
+    second time so that the test knows where the runs of tiles begin)."""
+    s = 1
+    while s < 32 and 2 * s * 16 <= n_tiles:
+        s *= 2
+    return s
+
+
+@pytest.mark.parametrize("kv, window", [(1100, None), (2500, None), (9000, None), (9000, 5000)])
+def test_decode_attention_finds_one_far_key_however_its_runs_are_spread(hip, kv, window):
+    """A decoding sequence of 1,100 to 9,000 keys is cut into 2 to 16 splits of four runs of tiles each, and the
+    runs are spread over workgroups in three ways: a workgroup a run (few sequences), a workgroup a split (some),
+    one workgroup for all of a sequence's runs (a crowd).  One key is made to stand out and the output must be its
+    value row, with the key at the first and the last position of runs in the middle of a split, at a split's
+    edge, in the very first and the very last run, and on either side of a window's edge; in each of the three ways,
+    and in a grid sized for a longer sequence than the step holds."""
+    n_heads, n_kv, D, ps = 4, 2, 64, 16
+    dtype = torch.bfloat16
+    lib = hip._attn_lib(D)
+    last = kv - 1
+    lo_all = max(0, last - window + 1) if window else 0
+    t_first, n_tiles = lo_all // 32, last // 32 - lo_all // 32 + 1
+    n_splits = _decode_splits(n_tiles)
+    n_runs = 4 * n_splits
+    assert n_splits >= 2
+    begin = lambda run: (t_first + run * n_tiles // n_runs) * 32         # first key of a run
+    runs = sorted({1, 2, 4, 5, n_runs // 2, n_runs - 4, n_runs - 1})
+    places = {max(lo_all, begin(run)) for run in runs} | {begin(run) - 1 for run in runs if begin(run) - 1 >= lo_all}
+    cases = [(p, True) for p in sorted(places | {lo_all, last})]
+    if window:
+        cases += [(lo_all - 1, False), (lo_all + 1, True)]
+    n_pages = -(-kv // ps)
+    direction = torch.nn.functional.normalize(rnd(D, seed=3), dim=0)
+    base_k = (0.01 * rnd(n_pages, n_kv, ps, D, seed=1)).to(dtype)
+    cache = Cache(n_pages, n_kv, ps, D, dtype, [kv], seed=5)
+    cache.v_pages.copy_(rnd(n_pages, n_kv, D, ps, seed=2).to(dtype))
+    row = cache.block_table[0].clone()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    crowd = -(-cus // n_kv) + 3                                            # a (sequence, kv head) pair a compute unit
+    some = -(-cus // (n_kv * n_splits)) + 1                                # more splits than compute units
+    seen_modes = set()
+    for n_seqs, bound, want_mode in ((1, 0, 2), (some, 0, 0), (crowd, 0, 1), (1, 4 * kv, 2), (crowd, 2 * kv, 1)):
+        ctx = Ctx([1] * n_seqs, [kv] * n_seqs)
+        ctx.kv_bound = bound
+        max_splits = lib.sia_attn_decode_max_splits(bound or kv, window or 0)
+        if some * n_kv >= cus and want_mode == 0:
+            continue                                                       # two splits only: no step takes that way
+        assert lib.sia_attn_decode_mode(n_seqs, n_heads, n_kv, max_splits) == want_mode, (n_seqs, bound)
+        seen_modes.add(want_mode)
+        cache.block_table = row.repeat(n_seqs, 1).contiguous()             # every sequence reads the same pages
+        qkv = torch.zeros(n_seqs, (n_heads + 2 * n_kv) * D)
+        qkv[:, :n_heads * D] = (30.0 * direction).repeat(n_heads)
+        qkv = qkv.to(dtype).to(DEV)
+        for far, seen in cases:
+            cache.k_pages.copy_(base_k)
+            page = int(row[far // ps])
+            cache.k_pages[page, :, far % ps] = (30.0 * direction).to(dtype)
+            out = hip.paged_attention(qkv, n_heads, n_kv, D, 1 / math.sqrt(D), window, ctx, cache).float()
+            for s in sorted({0, n_seqs // 2, n_seqs - 1}):
+                got = out[s].view(n_heads, D)
+                for h in range(n_heads):
+                    want = cache.v_pages[page, h // 2, :, far % ps].float()
+                    assert torch.allclose(got[h], want, rtol=2e-2, atol=2e-2) == seen, (n_seqs, bound, far, s, h)
+    assert {1, 2} <= seen_modes
 
 
 @pytest.mark.parametrize("vocab", [16, 1000, 128256])

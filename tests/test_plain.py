@@ -294,3 +294,27 @@ def test_sampling_by_inverse_cdf():
     assert torch.allclose(counts / 4000, torch.softmax(small / 0.7, -1), atol=0.03)
     only = plain.sample_with_uniform(small, 0.9, temperature=1.0, top_k=1)
     assert only == 2
+
+
+def test_the_model_with_the_references_roundings_is_the_model_when_nothing_is_rounded(tmp_path):
+    """``forward_as_the_reference_rounds`` composes the same part functions; with a rounding that does nothing it is
+    ``forward``, and with bfloat16 roundings it lies near it, further for more layers."""
+    from helpers import TINIES, random_tokens, rel_err, write_tiny_model
+    import copy
+    tiny = TINIES["b"]
+    folder = write_tiny_model(tmp_path / "b", tiny, seed=3)
+    cfg, w = plain.read_model(folder, torch.float64)
+    tokens = random_tokens(cfg["vocab_size"], 40, seed=1)
+    exact = plain.forward(cfg, w, tokens)
+    same = plain.forward_as_the_reference_rounds(cfg, w, tokens, rnd=lambda t: t)
+    assert torch.equal(same, exact)
+    rows = plain.forward_as_the_reference_rounds(cfg, w, tokens, rows=[3, 39], rnd=lambda t: t)
+    assert torch.allclose(rows, exact[[3, 39]], rtol=0, atol=1e-12)     # a product of 2 rows sums in another order
+    rounded = plain.forward_as_the_reference_rounds(cfg, w, tokens)
+    assert 1e-4 < rel_err(rounded, exact) < 2.5e-2
+    deep = copy.deepcopy(tiny.config)
+    deep["num_hidden_layers"] = 12
+    folder = write_tiny_model(tmp_path / "deep", tiny, seed=3, config=deep)
+    cfg12, w12 = plain.read_model(folder, torch.float64)
+    exact12 = plain.forward(cfg12, w12, tokens)
+    assert rel_err(plain.forward_as_the_reference_rounds(cfg12, w12, tokens), exact12) > rel_err(rounded, exact)

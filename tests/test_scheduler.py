@@ -402,3 +402,29 @@ def test_the_engine_goes_on_eagerly_when_its_graphs_give_up(folder, capsys):
     assert "replay refused" in capsys.readouterr().err
     eng.cache.check()
     assert eng.cache.free_pages() == eng.cfg.resolved_num_kv_blocks()
+
+
+def test_generate_takes_text_where_the_folder_has_a_tokenizer(tmp_path):
+    """Reference: ``generate.py:50-119`` takes the prompt as text and yields pieces of text.  The same request given
+    as token ids yields the ids those pieces decode from."""
+    from tokenizers import Tokenizer as Fast
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import Whitespace
+    folder = write_tiny_model(tmp_path, TINIES["a"], seed=11)
+    words = {f"w{i}": i for i in range(256)}
+    fast = Fast(WordLevel(words, unk_token="w0"))
+    fast.pre_tokenizer = Whitespace()
+    fast.save(str(tmp_path / "tokenizer.json"))
+    eng = engine(folder, block_size=4)
+    text = "w17 w5 w200 w33"
+    ids = [TINIES["a"].config["bos_token_id"], 17, 5, 200, 33]
+    assert eng.tokenizer().encode(text) == ids
+    by_ids = list(eng.generate(ids, max_new_tokens=6, temperature=0.0))
+    pieces = list(eng.generate(text, max_new_tokens=6, temperature=0.0))
+    assert "".join(pieces) == eng.tokenizer().decode(by_ids) and len(pieces) == len(by_ids)
+    out, stats = eng.generate_with_stats(text, max_new_tokens=6, temperature=0.0)
+    assert out == "".join(pieces) and stats["prompt_tokens"] == 5
+    other = Engine.from_random(TINIES["a"].config, 0, EngineConfig(device="cpu", dtype="float32", max_seq_len=64,
+                                                                  use_graphs=False), TwinKernels())
+    with pytest.raises(ValueError, match="token ids"):
+        next(other.generate("w1 w2"))

@@ -106,3 +106,46 @@ def test_untied_head_is_a_tensor_of_its_own(tmp_path):
     folder = write_tiny_model(tmp_path / "tied", TINIES["a"], seed=2)
     model, _ = model_from_folder(folder, EngineConfig(device="cpu", dtype="float32", max_seq_len=64), TwinKernels())
     assert model.head.weight.data_ptr() == model.embedding.weight.data_ptr()     # tied: same storage
+
+
+def test_a_tied_model_stored_with_its_head_is_taken_if_the_head_repeats_the_embedding(tmp_path):
+    """The reference reads an ``lm_head.weight`` that a tied checkpoint also stores (``model/llama.py:147-154``).
+    Here it is passed over when it repeats the embedding, and refused with both names when it does not: the
+    configuration says one matrix, the file holds two."""
+    from twins import TwinKernels
+    from simple_inference_amd.engine import model_from_folder
+    ecfg = EngineConfig(device="cpu", dtype="float32", max_seq_len=64)
+    exp = expected_of(TINY_A)
+    t = random_tensors(exp, 3)
+    t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
+    write_model_folder(tmp_path / "same", TINY_A, t)
+    model, _ = model_from_folder(tmp_path / "same", ecfg, TwinKernels())
+    assert model.head.weight.data_ptr() == model.embedding.weight.data_ptr()
+    t["lm_head.weight"][3, 5] += 1.0
+    write_model_folder(tmp_path / "other", TINY_A, t)
+    with pytest.raises(WeightError, match="lm_head.weight is not equal to model.embed_tokens.weight") as e:
+        model_from_folder(tmp_path / "other", ecfg, TwinKernels())
+    assert e.value.differing == [("lm_head.weight", "model.embed_tokens.weight")] and not e.value.unexpected
+    t["lm_head.weight"] = torch.zeros(3, 64, dtype=torch.bfloat16)
+    write_model_folder(tmp_path / "shape", TINY_A, t)
+    with pytest.raises(WeightError) as e:
+        model_from_folder(tmp_path / "shape", ecfg, TwinKernels())
+    assert e.value.wrong_shape == [("lm_head.weight", (3, 64), (256, 64))]
+    # an untied model has a head of its own: nothing there may be stored twice
+    model, _ = build_model(TINY_B, ecfg, kernels=None)
+    assert model.plan.duplicates == {}
+
+
+def test_the_parts_hold_as_many_parameters_as_the_configuration_counts():
+    """Reference: ``loader.py:301-316`` checks the loaded total against the model's known size."""
+    from simple_inference_amd import preset
+    from simple_inference_amd.engine.build import count_parameters, describe
+    ecfg = EngineConfig(device="cpu", dtype="bfloat16", max_seq_len=64)
+    for name, total in (("llama-3.2-3b", 3_212_749_824), ("llama-3.2-1b", 1_235_814_400), ("llama-3.1-8b", 8_030_261_248)):
+        model, cfg = build_model(preset(name), ecfg, kernels=None)
+        assert count_parameters(model, cfg) == total
+    assert "3,212,749,824 parameters" not in describe(model, cfg, ecfg) and "131,072 bytes of cache a token" in describe(model, cfg, ecfg)
+    model, cfg = build_model(TINY_B, ecfg, kernels=None)
+    object.__setattr__(cfg, "intermediate_size", cfg.intermediate_size + 1)
+    with pytest.raises(ValueError, match="formula"):
+        count_parameters(model, cfg)

@@ -81,3 +81,39 @@ def test_more_rows_than_the_array_holds_are_refused():
                                  torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert code == REFUSED and out.tolist() == [-1] * rows
+
+
+def test_recorded_into_a_graph_after_the_address_was_looked_up_outside_it():
+    """The look-up of the array's address is no stream operation: ``sia_sample_static_init`` does it before the
+    recording starts, and the recorded call then only launches kernels.  The graph is replayed several times on
+    new inputs, with eager work and waits between the replays, and every replay gives the eager call's tokens."""
+    lib = _library()
+    lib.sia_sample_static_init.argtypes, lib.sia_sample_static_init.restype = [], ctypes.c_int
+    assert lib.sia_sample_static_init() == 0
+    rows, vocab = 6, 4099
+    logits, temperature, top_k, top_p, uniform = _case(rows, vocab, seed=20)
+    out = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+    ptr = lambda t: t.data_ptr()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            code = lib.sia_sample_static(ptr(logits), ptr(temperature), ptr(top_k), ptr(top_p), ptr(uniform), ptr(out),
+                                         rows, vocab, 7, torch.cuda.current_stream().cuda_stream)
+    assert code == 0
+    torch.cuda.current_stream().wait_stream(side)
+    for seed in (21, 22, 23):
+        fresh = _case(rows, vocab, seed)
+        for dst, src in zip((logits, temperature, top_k, top_p, uniform), fresh):
+            dst.copy_(src)
+        out.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.tolist()
+        want = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        workspace = torch.zeros(lib.sia_sample_workspace_bytes(rows), dtype=torch.uint8, device=DEV)
+        assert lib.sia_sample(ptr(logits), ptr(temperature), ptr(top_k), ptr(top_p), ptr(uniform), ptr(want),
+                              ptr(workspace), rows, vocab, 7, torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        assert got == want.tolist(), seed
