@@ -45,3 +45,8 @@ def test_decode_allowance_covers_the_steps_that_build_the_contexts():
     assert bench.decode_allowance(2048, 8, 2048) == 8 + 2
     assert bench.decode_allowance(2048, 8, 8192) == 8 * 4 + 2
     assert bench.decode_allowance(2048, 64, 2049) == 64 * 2 + 2
+
+
+def test_the_bound_on_the_logits_is_the_measured_one_at_the_headline_depth():
+    import bench
+    assert bench.logit_bound(28) == 5.0e-2 and 1.3e-2 < bench.logit_bound(2) < 1.4e-2
