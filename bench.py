@@ -61,7 +61,10 @@ def parse_args(argv=None):
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--block-size", type=int, default=None)
     ap.add_argument("--no-graphs", action="store_true")
-    ap.add_argument("--points", default="1,64", help="further decode batch sizes to report, comma separated")
+    ap.add_argument("--points", default="1,64,16,17", help="further decode batch sizes to report, comma separated")
+    ap.add_argument("--no-further-points", action="store_true",
+                    help="only the headline and --points: no long contexts, other prompt lengths or request streams")
+    ap.add_argument("--chunk-tokens", type=int, default=512, help="most tokens a step of the stream workloads runs")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-check", action="store_true", help="skip the comparison of logits with the float32 engine")
     ap.add_argument("--seed", type=int, default=0)
@@ -197,11 +200,12 @@ def logits_check(engine, cfg, seed, batch=4, context=512):
             "ok": bool(rel <= bound and ties)}
 
 
-def run_stream(preset_name, requests, max_running, max_seq_len, prefix_cache, args):
+def run_stream(preset_name, requests, max_running, max_seq_len, prefix_cache, args, chunk_tokens=None):
     """Queues all requests at once and steps the engine dry; returns the figures of the run."""
     from simple_inference_amd import Engine, EngineConfig, SamplingParams, preset
 
-    ecfg = EngineConfig(max_running=max_running, max_seq_len=max_seq_len, chunk_tokens=512, dtype=args.dtype,
+    ecfg = EngineConfig(max_running=max_running, max_seq_len=max_seq_len,
+                        chunk_tokens=chunk_tokens or args.chunk_tokens, dtype=args.dtype,
                         eos_id=-1, use_graphs=not args.no_graphs, use_prefix_cache=prefix_cache, device="cuda:0")
     engine = Engine.from_random(preset(preset_name), seed=args.seed, engine_cfg=ecfg, std=0.02,
                                 generate_on_device=True)
@@ -276,35 +280,104 @@ def stream_check(engine, finished, sample=4, last=8):
     return {"requests": len(picks), "tokens": total, "same_as_solo": same, "tied_within_rounding": close - same}
 
 
-def stream_workload(args):
+def continuous_requests(seed):
+    """128 requests of the 1B workload: prompts of 64..2,048 and outputs of 32..512 tokens, uniform."""
     import random
 
     from simple_inference_amd import preset
+    rng = random.Random(seed)
+    vocab = preset("llama-3.2-1b")["vocab_size"]
+    return [([rng.randrange(vocab) for _ in range(rng.randint(64, 2048))], rng.randint(32, 512)) for _ in range(128)]
 
-    rng = random.Random(args.seed)
+
+def shared_prefix_requests(seed):
+    """64 requests of the 8B workload: one 1,024-token prefix, 256 tokens of their own, 256 decoded tokens each."""
+    import random
+
+    from simple_inference_amd import preset
+    rng = random.Random(seed)
+    vocab = preset("llama-3.1-8b")["vocab_size"]
+    shared = [rng.randrange(vocab) for _ in range(1024)]
+    return [(shared + [rng.randrange(vocab) for _ in range(256)], 256) for _ in range(64)]
+
+
+def stream_workload(args):
     if args.workload == "continuous":
         name = "llama-3.2-1b"
-        vocab = preset(name)["vocab_size"]
-        requests = [([rng.randrange(vocab) for _ in range(rng.randint(64, 2048))], rng.randint(32, 512))
-                    for _ in range(128)]
-        run = run_stream(name, requests, args.max_running, 4096, False, args)
+        run = run_stream(name, continuous_requests(args.seed), args.max_running, 4096, False, args)
         line = {"metric": "generated tok/s, continuous batching of 128 requests (1B shape)", "value": run["generated_tok_s"],
                 "run": run}
     else:
         name = "llama-3.1-8b"
-        vocab = preset(name)["vocab_size"]
-        shared = [rng.randrange(vocab) for _ in range(1024)]
-        requests = [(shared + [rng.randrange(vocab) for _ in range(256)], 256) for _ in range(64)]
+        requests = shared_prefix_requests(args.seed)
         reuse = run_stream(name, requests, args.max_running, 8192, True, args)
         plain = run_stream(name, requests, args.max_running, 8192, False, args)
         line = {"metric": "generated tok/s, 64 requests with a shared 1,024-token prefix (8B shape), prefix reuse on",
                 "value": reuse["generated_tok_s"], "run": reuse, "without_reuse": plain}
     line.update({"unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "warmup": "one untimed pass of the same stream", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
                  "data": "synthetic (seeded random weights N(0, 0.02) and uniform-random token ids)",
-                 "config": {"model": name + "-shape", "max_running": args.max_running, "chunk_tokens": 512,
+                 "config": {"model": name + "-shape", "max_running": args.max_running, "chunk_tokens": args.chunk_tokens,
                             "graphs": not args.no_graphs}})
     print(json.dumps(line), flush=True)
     return 0
+
+
+def further_points(args, pts, config, layer_w, head_w, el):
+    """What the headline leaves out, at sizes a server meets: the same model with contexts of 8,192 and 32,768 tokens
+    and a prompt of 8,192 (an engine of its own with a context limit of 33,792), and the two request streams of the
+    other shapes, each through scheduler, step function and sampler, with a sample of its tokens checked against
+    solo runs."""
+    import copy
+    from simple_inference_amd import Engine, EngineConfig, preset
+
+    long_args = copy.copy(args)
+    long_limit = 32768 + 1024
+    cfg = preset(args.preset)
+    if args.layers is not None:
+        cfg["num_hidden_layers"] = args.layers
+    steps, warmup = min(args.steps, 32), min(args.warmup, 4)
+    ecfg = EngineConfig(max_running=8, max_seq_len=long_limit, dtype=args.dtype, chunk_tokens=8192, eos_id=-1,
+                        use_graphs=not args.no_graphs, device="cuda:0")
+    ecfg.num_kv_blocks = 8 * (-(-long_limit // ecfg.block_size)) + 8
+    engine = Engine.from_random(cfg, seed=args.seed, engine_cfg=ecfg, std=0.02, generate_on_device=True)
+    mc = engine.model_cfg
+    config["long_context_limit"] = long_limit
+    for context in (8192, 32768):
+        dt, ctx = measure_decode(engine, 8, context, steps, warmup, args.seed)
+        gbs = ((layer_w + head_w) * el + 8 * ctx * mc.kv_bytes_per_token(el)) / dt / 1e9
+        pts[f"decode_b8_ctx{context}"] = round(8 / dt, 2)
+        pts[f"decode_b8_ctx{context}_hbm_frac"] = round(gbs / PEAK_HBM_GBS, 4)
+    if not args.no_prefill:
+        T = 8192
+        sec, _ = measure_prefill(engine, T, repeats=2)
+        flops = 2 * layer_w * T + 2 * head_w + mc.num_hidden_layers * 4 * mc.num_attention_heads * mc.head_dim * T * (T + 1) / 2
+        pts["prefill_8192"] = round(T / sec, 1)
+        pts["prefill_8192_frac"] = round(flops / sec / PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"], 4)
+    del engine
+    torch.cuda.empty_cache()
+    if args.preset != "llama-3.2-3b" or args.layers is not None:
+        return      # the streams belong to the default run
+    run = run_stream("llama-3.2-1b", continuous_requests(args.seed), 64, 4096, False, args)
+    config["stream_1b"] = f"llama-3.2-1b-shape, 128 requests, max_running 64, chunk_tokens {args.chunk_tokens}"
+    pts["stream_1b_tok_s"] = run["generated_tok_s"]
+    pts["stream_1b_seconds"] = run["seconds"]
+    pts["stream_1b_tpot_p50_ms"] = run["tpot_ms"]["p50"]
+    pts["stream_1b_tpot_p99_ms"] = run["tpot_ms"]["p99"]
+    pts["stream_1b_checked_tokens"] = run["check"]["tokens"]
+    # the same stream with portions of 2,048 tokens: fewer, fuller steps (a step of 512 rows costs 1.8 times as much a
+    # token as one of 2,048), paid for by the decoding requests that wait behind them
+    wide = run_stream("llama-3.2-1b", continuous_requests(args.seed), 64, 4096, False, args, chunk_tokens=2048)
+    pts["stream_1b_chunk2048_tok_s"] = wide["generated_tok_s"]
+    pts["stream_1b_chunk2048_tpot_p50_ms"] = wide["tpot_ms"]["p50"]
+    pts["stream_1b_chunk2048_tpot_p99_ms"] = wide["tpot_ms"]["p99"]
+    requests = shared_prefix_requests(args.seed)
+    config["prefix_8b"] = f"llama-3.1-8b-shape, 64 requests, prefix 1024, max_running 64, chunk_tokens {args.chunk_tokens}"
+    reuse = run_stream("llama-3.1-8b", requests, 64, 8192, True, args)
+    plain = run_stream("llama-3.1-8b", requests, 64, 8192, False, args)
+    pts["prefix_8b_seconds"] = reuse["seconds"]
+    pts["prefix_8b_seconds_without"] = plain["seconds"]
+    pts["prefix_8b_prompt_tokens_run"] = reuse["prefill_tokens_run"]
+    pts["prefix_8b_checked_tokens"] = reuse["check"]["tokens"] + plain["check"]["tokens"]
 
 
 def main(argv=None):
@@ -369,10 +442,18 @@ def main(argv=None):
         _, p_tok_s, p_gbs = decode_point(b)
         pts[f"decode_b{b}"] = round(p_tok_s, 2)
         pts[f"decode_b{b}_hbm_frac"] = round(p_gbs / PEAK_HBM_GBS, 4)
-    if pts:
-        line["points"] = pts
     if not args.no_check and args.dtype == "bfloat16":
         line["check"] = logits_check(engine, cfg, args.seed)
+    if not args.no_further_points and not args.no_prefill:
+        sec, _ = measure_prefill(engine, 512)        # the default portion of a prompt (chunk_tokens of the engine)
+        pts["prefill_512"] = round(512 / sec, 1)
+        pts["prefill_512_ms"] = round(sec * 1e3, 3)
+    if not args.no_further_points:
+        del engine
+        torch.cuda.empty_cache()
+        further_points(args, pts, line["config"], layer_w, head_w, el)
+    if pts:
+        line["points"] = pts
     print(json.dumps(line), flush=True)
     if "check" in line and not line["check"]["ok"]:
         print(f"bench.py: the bfloat16 logits are further from the float32 engine's than a correct bfloat16 "
