@@ -189,23 +189,26 @@ SIA_EXPORT int sia_blas_mm(const void* X, const void* W, void* Y, int M, int N, 
     State* st = state_of_current_device();
     if (!st) return 1;
     if (M <= 0 || N <= 0 || K <= 0) return 2;
-    const uint64_t key = ((uint64_t)(uint32_t)M << 42) ^ ((uint64_t)(uint32_t)N << 21) ^ (uint64_t)(uint32_t)K ^
-                         ((uint64_t)(out_float ? 1 : 0) << 63);
-    // Candidates are timed only while the caller says that the shapes it runs will recur, and never while the stream
-    // is being captured into a graph (a graph's shapes are met in the eager runs before its capture).
+    // Plans chosen by timing are kept apart from the library's first choices (bit 62 of the key) and are used only
+    // while the caller says that the shapes it runs will recur: the runs before a graph is captured and the capture
+    // itself.  Every other call takes the first choice, so a product outside a graph never changes its algorithm
+    // (and with it the last bits of its result) because some graph was captured in between.  Candidates are never
+    // timed while the stream is being captured (a graph's shapes are met in the eager runs before its capture).
+    const bool tuned = st->try_out && M <= TRY_OUT_ROWS;
+    uint64_t key = ((uint64_t)(uint32_t)M << 42) ^ ((uint64_t)(uint32_t)N << 21) ^ (uint64_t)(uint32_t)K ^
+                   ((uint64_t)(out_float ? 1 : 0) << 63) ^ ((uint64_t)(tuned ? 1 : 0) << 62);
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    const bool try_out = st->try_out && M <= TRY_OUT_ROWS && hipStreamIsCapturing(stream, &capturing) == hipSuccess &&
-                         capturing == hipStreamCaptureStatusNone;
+    const bool may_time = tuned && hipStreamIsCapturing(stream, &capturing) == hipSuccess &&
+                          capturing == hipStreamCaptureStatusNone;
     auto it = st->plans.find(key);
-    if (it == st->plans.end() || (try_out && !it->second.tried_out)) {
+    if (it == st->plans.end() && tuned && !may_time) {   // captured without a timed run before it: the first choice
+        key ^= (uint64_t)1 << 62;
+        it = st->plans.find(key);
+    }
+    if (it == st->plans.end()) {
         Plan p;
-        make_plan(*st, p, M, N, K, out_float != 0, try_out, X, W, Y, stream);
-        if (it != st->plans.end()) {
-            release(it->second);
-            it->second = p;
-        } else {
-            it = st->plans.emplace(key, p).first;
-        }
+        make_plan(*st, p, M, N, K, out_float != 0, may_time, X, W, Y, stream);
+        it = st->plans.emplace(key, p).first;
     }
     const Plan& p = it->second;
     if (!p.ok) return 3;

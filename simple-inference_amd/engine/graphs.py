@@ -203,7 +203,7 @@ class GraphedDecode:
         collecting = gc.isenabled()
         gc.disable()   # no destructor of an older graph may run while the stream is capturing
         try:
-            with torch.cuda.graph(graph):
+            with settle(), torch.cuda.graph(graph):   # records the algorithms the runs above settled on
                 b.logits = model.forward(b.ctx, b.caches)
         finally:
             if collecting:

@@ -181,8 +181,11 @@ class HipKernels:
     @contextlib.contextmanager
     def recurring_shapes(self):
         """Inside, the products that go to the BLAS library have the library's candidate algorithms timed on their
-        own operands when their shape is first met (few rows only), and the fastest kept.  For runs whose shapes will
-        recur many times: the eager runs before a graph is captured."""
+        own operands when their shape is first met (few rows only), and the fastest kept, for use inside this context
+        only: products outside it keep the library's first choice.  For runs whose shapes will recur many times: the
+        eager runs before a graph is captured, and the capture itself (which times nothing and records what those
+        runs chose).  Which candidate wins is decided by the clock, so the last bits of a replayed step's products
+        can differ from one process to the next; within a process a graph, once captured, never changes."""
         if self.blas is None:
             yield
             return

@@ -77,28 +77,33 @@ def test_graph_replay_equals_eager_on_every_replay(folders, dtype):
 def test_graph_replay_of_many_rows_equals_eager_on_every_replay(folders):
     """Twenty and more requests: the products of a replayed step then go to the BLAS library, whose launches are
     captured with this package's.  Every replay's logits against the same step run eagerly on a twin engine, with
-    eager work and synchronisation between the replays (a captured memset would show from the second replay on)."""
+    eager work and synchronisation between the replays (a captured memset would show from the second replay on).
+    The eager twin runs where a graph's shapes are settled (``recurring_shapes``), so that it multiplies with the
+    library algorithms the graph recorded: the same kernels and library calls, replayed or not, give the same
+    bits.  Outside that context an eager step keeps the library's first choice and may differ in the last bits."""
     tiny = TINIES["d"]
     vocab = tiny.config["vocab_size"]
     kw = dict(max_running=24, max_seq_len=128, chunk_tokens=64, run_ahead=False)
     eager = engine(folders["d"], tiny, "bfloat16", use_graphs=False, **kw)
     graphed = engine(folders["d"], tiny, "bfloat16", use_graphs=True, **kw)
-    prompts = [random_tokens(vocab, 3 + (7 * i) % 19, seed=120 + i) for i in range(22)]
+    prompts = [random_tokens(vocab, 3 + (7 * i) % 19, seed=120 + i) for i in range(24)]
     for eng in (eager, graphed):
         for i, p in enumerate(prompts):
             eng.cache.admit(i)
             eng.runner.run([StepEntry(i, p, [])])
-    tokens = [random_tokens(vocab, 12, seed=200 + i) for i in range(22)]
-    worst = 0.0
+    tokens = [random_tokens(vocab, 12, seed=200 + i) for i in range(24)]
     for step in range(12):
-        live = list(range(22 - step // 4))        # 22, 21, 20 rows: one bucket, other paddings
+        live = list(range(24 - step // 4))        # 24, 23, 22 rows: one bucket, full and with padding rows
         entries = [StepEntry(i, [tokens[i][step]], [0]) for i in live]
-        want = eager.runner.run(entries)
+        with eager.kernels.recurring_shapes():
+            want = eager.runner.run(entries)
         got = graphed.graphs.run(entries)
         torch.cuda.synchronize()
-        worst = max(worst, rel_err(got, want))
+        if len(live) == 24:      # the bucket's own number of rows: the library is asked for the same product
+            assert torch.equal(got, want), (step, rel_err(got, want))
+        else:                    # fewer rows run eagerly as a product of fewer rows, for which the library may choose otherwise
+            assert rel_err(got, want) <= 1e-2, (step, rel_err(got, want))
     assert graphed.graphs.replays == 12 and len(graphed.graphs._made) == 1
-    assert worst <= 1e-2, worst    # the same kernels and library calls, replayed or not
 
 
 def test_long_decoding_crosses_the_length_buckets_of_the_graphs(folders):
