@@ -106,6 +106,35 @@ def test_graph_replay_of_many_rows_equals_eager_on_every_replay(folders):
     assert graphed.graphs.replays == 12 and len(graphed.graphs._made) == 1
 
 
+def test_a_replayed_step_that_finds_no_page_leaves_the_books_as_they_were(folders):
+    """Requests admitted without a promise (as trace replay admits them) can run out of pages in the middle of a
+    step's bookkeeping: the first request of the step has been given its position, the second finds no page.  The
+    step then raises with every request as long as before, and runs once a page is free."""
+    from simple_inference_amd.cache.allocator import OutOfPages
+    tiny = TINIES["d"]
+    vocab, ps = tiny.config["vocab_size"], tiny.page_size
+    eng = engine(folders["d"], tiny, "bfloat16", use_graphs=True, max_seq_len=64, num_kv_blocks=3, run_ahead=False)
+    lengths = {1: ps - 1, 2: ps, 3: 5}        # request 2 fills its page exactly: its next token needs a new one
+    for rid, n in lengths.items():
+        eng.cache.admit(rid)
+        eng.runner.run([StepEntry(rid, random_tokens(vocab, n, seed=rid), [])])
+    assert eng.cache.free_pages() == 0
+    entries = [StepEntry(1, [7], [0]), StepEntry(2, [8], [0])]
+    with pytest.raises(OutOfPages):
+        eng.graphs.run(entries)
+    assert {rid: eng.cache.lengths[rid] for rid in lengths} == lengths
+    eng.cache.check()
+    eng.cache.release(3)                      # a page comes back: the same step now runs
+    logits = eng.graphs.run(entries)
+    torch.cuda.synchronize()
+    assert logits.shape[0] == 2 and eng.cache.lengths[1] == ps and eng.cache.lengths[2] == ps + 1
+    eager = engine(folders["d"], tiny, "bfloat16", use_graphs=False, max_seq_len=64, num_kv_blocks=3)
+    for rid in (1, 2):
+        eager.cache.admit(rid)
+        eager.runner.run([StepEntry(rid, random_tokens(vocab, lengths[rid], seed=rid), [])])
+    assert torch.equal(logits, eager.runner.run(entries))
+
+
 def test_long_decoding_crosses_the_length_buckets_of_the_graphs(folders):
     """Decoding from 500 to 1,040 tokens of context: the replayed graphs change from the 512-token bucket to the
     1,024-token one and on to the last (other attention grids and key splits), and every token stays the one an
