@@ -610,8 +610,12 @@ class HipKernels:
         if forms is not None:
             return forms
         block.plain_forms = False
-        parts = [getattr(p, "plain_form", lambda: None)()
-                 for p in (block.mixer_norm, block.mixer, block.feed_forward_norm, block.feed_forward)]
+        # the block says what it is: its kind and its parts' own descriptions.  The one-call form exists for a
+        # pre-norm block of an RMS norm, paged attention, an RMS norm and a SwiGLU feed-forward.
+        whole = getattr(block, "plain_form", lambda: None)()
+        if not whole or whole.get("kind") != "prenorm":
+            return False
+        parts = [whole.get(name) for name in ("mixer_norm", "mixer", "feed_forward_norm", "feed_forward")]
         if any(f is None for f in parts) or [f["kind"] for f in parts] != ["rmsnorm", "paged_attention", "rmsnorm", "swiglu"]:
             return False
         n1, at, n2, ff = parts

@@ -20,9 +20,19 @@ class PreNormBlock:
         self.feed_forward_norm = feed_forward_norm
         self.plain_forms = None   # kept by kernels that run the block in one call: what they made of the parts
 
+    def plain_form(self):
+        """What this block is, as plain data, for kernels that can make all of its launches in one call: its kind
+        (the order in which the parts run is this file's affair: the docstring above) and what each part says it is
+        (its own ``plain_form``; None for a part that has none, and such a block goes part by part)."""
+        if type(self).forward is not PreNormBlock.forward:
+            return None
+        form = lambda part: getattr(part, "plain_form", lambda: None)()
+        return {"kind": "prenorm", "mixer_norm": form(self.mixer_norm), "mixer": form(self.mixer),
+                "feed_forward_norm": form(self.feed_forward_norm), "feed_forward": form(self.feed_forward)}
+
     def forward(self, stream, ctx, cache):
-        # Kernels that can make all of a block's launches in one call are shown the block (they look at what its
-        # parts say they are, ``plain_form``, and take it or leave it); else part by part.
+        # Kernels that can make all of a block's launches in one call are shown the block (they look at what it and
+        # its parts say they are, ``plain_form``, and take it or leave it); else part by part.
         whole = getattr(ctx.kernels, "prenorm_block", None)
         if whole is not None and whole(self, stream, ctx, cache):
             return

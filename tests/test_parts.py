@@ -181,3 +181,50 @@ def test_embedding_and_head_parts(backend):
     untied = OutputHead({"vocab_size": 331, "hidden_size": 40, "tied": False}, env)
     untied.bind({"weight": on(env, own)})
     assert rel_err(untied.forward(on(env, h)), as_ref(env, h) @ as_ref(env, own).T) <= tol(backend)
+
+
+def test_a_part_with_a_forward_of_its_own_no_longer_says_it_is_the_plain_one():
+    """Kernels that run a whole block in one call trust what the block and its parts say they are (``plain_form``).
+    A subclass that computes something else (a forward of its own) must not inherit that description, or steps of
+    many rows would silently run the base class's arithmetic while steps of few rows run the subclass's."""
+    from simple_inference_amd.parts.attention import Attention
+    from simple_inference_amd.parts.block import PreNormBlock
+    from simple_inference_amd.parts.norm import RMSNorm
+    from simple_inference_amd.parts.swiglu import SwiGLU
+    env = env_for("twins")
+    rope = {"kind": "rope", "params": {"rotary_dim": 16, "theta": 10000.0, "scaling": None}}
+    attn_params = {"hidden_size": 32, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16, "position": rope}
+
+    class OtherAttention(Attention):
+        def forward(self, h, ctx, cache):
+            return 2 * super().forward(h, ctx, cache)
+
+    class OtherNorm(RMSNorm):
+        def forward(self, stream, rows=None, scaled_ok=False):
+            return super().forward(stream, rows) + 1
+
+    class OtherFeedForward(SwiGLU):
+        def forward(self, h, ctx):
+            return -super().forward(h, ctx)
+
+    class OtherBlock(PreNormBlock):
+        def forward(self, stream, ctx, cache):
+            super().forward(stream, ctx, cache)
+
+    def built(attn_cls, norm_cls, ff_cls, block_cls):
+        mixer, ff = attn_cls(attn_params, env), ff_cls({"hidden_size": 32, "intermediate_size": 48}, env)
+        n1, n2 = norm_cls({"size": 32, "eps": 1e-5}, env), norm_cls({"size": 32, "eps": 1e-5}, env)
+        mixer.bind({k: rnd(*spec.shape, seed=1) for k, spec in mixer.weight_specs().items()})
+        ff.bind({k: rnd(*spec.shape, seed=2) for k, spec in ff.weight_specs().items()})
+        for n in (n1, n2):
+            n.bind({"weight": torch.ones(32)})
+        return block_cls(mixer=mixer, feed_forward=ff, mixer_norm=n1, feed_forward_norm=n2)
+
+    whole = built(Attention, RMSNorm, SwiGLU, PreNormBlock).plain_form()
+    assert whole["kind"] == "prenorm"
+    assert [whole[k]["kind"] for k in ("mixer_norm", "mixer", "feed_forward_norm", "feed_forward")] == \
+        ["rmsnorm", "paged_attention", "rmsnorm", "swiglu"]
+    assert built(OtherAttention, RMSNorm, SwiGLU, PreNormBlock).plain_form()["mixer"] is None
+    assert built(Attention, OtherNorm, SwiGLU, PreNormBlock).plain_form()["mixer_norm"] is None
+    assert built(Attention, RMSNorm, OtherFeedForward, PreNormBlock).plain_form()["feed_forward"] is None
+    assert built(Attention, RMSNorm, SwiGLU, OtherBlock).plain_form() is None
