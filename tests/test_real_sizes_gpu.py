@@ -335,3 +335,37 @@ def test_the_four_cuts_at_full_depth(full_depth, dtype):
     for r in (~same).nonzero().flatten().tolist():
         gap = float(exact[r].max() - exact[r, int(mine[r].argmax())])
         assert gap <= 2 * allowed_worst * scale, f"place {r}: best token differs and is no tie (gap {gap:.4f})"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_of_a_long_prompt_are_read_again_by_a_short_one_at_8b_widths(models, dtype):
+    """Prefix reuse at real widths: a prompt of 2,048 tokens fills its pages in one step of 2,048 rows (the library's
+    products, the prefill attention shape for long prompts, rotation and cache write of long steps); a second
+    request with the same first 1,024 tokens and 17 of its own then runs those 17 rows only, reading 64 pages the
+    first one wrote, and goes on decoding.  Its tokens are the plain implementation's (which knows no cache),
+    apart from ties within rounding in bfloat16."""
+    from simple_inference_amd import Engine, EngineConfig
+    folder, cfg, w = models("8b")
+    vocab = cfg["vocab_size"]
+    first = random_tokens(vocab, 2048, seed=500)
+    second = first[:1024] + random_tokens(vocab, 17, seed=501)
+    engine = Engine.from_folder(folder, EngineConfig(
+        device="cuda:0", dtype=dtype, max_seq_len=2304, block_size=PAGE, max_running=2, chunk_tokens=2048, eos_id=-1,
+        use_prefix_cache=True))
+    a = engine.add_request(first, max_new_tokens=2)
+    engine.run()
+    b = engine.add_request(second, max_new_tokens=6)
+    engine.run()
+    assert a.cached_prefix_len == 0 and b.cached_prefix_len == 1024
+    assert engine.stats["prefill_tokens"] == 2048 + 17
+    tolerance = TOLERANCE["hip-f32" if dtype == "float32" else "hip-bf16"]
+    w = {k: v.to("cuda:0") for k, v in w.items()}      # the plain implementation runs where its tensors lie
+    for req in (a, b):
+        tokens = list(req.prompt_tokens)
+        for got in req.generated:
+            logits = plain.forward(cfg, w, tokens, rows=[len(tokens) - 1])[0].cpu()
+            want = int(logits.argmax())
+            gap = float(logits[want] - logits[got])
+            assert got == want or (dtype == "bfloat16" and gap <= 2 * tolerance * float(logits.abs().max())), (got, want, gap)
+            tokens.append(got)
+    engine.cache.check()
