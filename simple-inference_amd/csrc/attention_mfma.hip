@@ -577,10 +577,12 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
 constexpr int PF_ROWS = HD <= 128 ? 128 : 64;  // tokens per wide workgroup
 constexpr int PF_ROWS_SPLIT = 64;              // tokens per split workgroup
 constexpr int PF_ROWS_LONG = 256;              // tokens per workgroup of 8 waves of 32 tokens
-// Key and value tiles are shared by the workgroup's waves through LDS (two stages).  Rows are padded by
-// 16 bytes so that the 16 lanes of a 128-bit read hit 64 different banks.
-constexpr int K_STRIDE = HD + 8;                // elements per key row
-constexpr int V_STRIDE = TILE + 8;              // elements per dim row (32 positions + pad)
+// Key and value tiles are shared by the workgroup's waves through LDS (two stages).  A 128-bit read takes the
+// 64 banks in four passes of 16 lanes, and the lanes of a pass are not neighbours: the first takes lanes 0-3,
+// 12-15, 20-23 and 24-27 (measured: rows of 16 lanes, one 16-byte piece each, are read without a conflict when the
+// rows lie an odd multiple of 32 bytes apart, and in twice the time when the row is padded by 16 bytes only).
+constexpr int K_STRIDE = HD + ((HD / 16) % 2 == 0 ? 16 : 0);  // elements per key row: an odd multiple of 32 bytes
+constexpr int V_STRIDE = TILE + 16;                           // elements per dim row (32 positions + pad): 96 bytes
 constexpr int K_CHUNKS = TILE * HD / 8;         // 16-byte pieces of a key tile (a value tile has as many)
 constexpr bool PF_USE_LDS = (2 * (TILE * K_STRIDE + HD * V_STRIDE) * 2) <= 64 * 1024;
 
@@ -620,13 +622,27 @@ struct FetchPlan {
     }
 };
 
-// Issues the global loads of the tile at kb.  Keys outside [lo, hi] are clamped into it (see load_stage); a key
-// piece and its value piece then still lie in one page: both are clamped into the same range, whose ends lie in
-// pages of their own only as a whole.  page_stride: elements of one page (keys and values alike).
+// The pages of a thread's pieces of the tile at kb, looked up a step before the tile's loads are issued, so that no
+// load's address waits for the exchange between lanes.  Keys outside [lo, hi] are clamped into it (see load_stage);
+// a key piece and its value piece then still lie in one page: both are clamped into the same range, whose ends lie
+// in pages of their own only as a whole.
+template <int TEAM>
+__device__ __forceinline__ void tile_lookup(int (&page)[TileRegs<TEAM>::PER_THREAD], const FetchPlan<TEAM>& plan,
+                                            const PageWindow& pages, int ps_log2, int kb, int lo, int hi) {
+    const int t_lo = max(kb, lo), t_hi = min(kb + TILE - 1, hi);
+#pragma unroll
+    for (int i = 0; i < TileRegs<TEAM>::PER_THREAD; ++i) {
+        const int key = min(max(kb + plan.k_key[i], t_lo), t_hi);
+        page[i] = pages_get(pages, key >> ps_log2);
+    }
+}
+
+// Issues the global loads of the tile at kb, whose pages tile_lookup found.  page_stride: elements of one page
+// (keys and values alike).
 template <int TEAM>
 __device__ __forceinline__ void tile_fetch(TileRegs<TEAM>& t, const FetchPlan<TEAM>& plan, const bf16_t* __restrict__ kp,
-                                           const bf16_t* __restrict__ vp, const PageWindow& pages, int ps_log2,
-                                           unsigned page_stride, int kb, int lo, int hi) {
+                                           const bf16_t* __restrict__ vp, const int (&page)[TileRegs<TEAM>::PER_THREAD],
+                                           int ps_log2, unsigned page_stride, int kb, int lo, int hi) {
     const int ps_mask = (1 << ps_log2) - 1;
     const int t_lo = max(kb, lo), t_hi = min(kb + TILE - 1, hi);
     const int v_lo = t_lo & ~7, v_hi = t_hi & ~7;
@@ -635,7 +651,7 @@ __device__ __forceinline__ void tile_fetch(TileRegs<TEAM>& t, const FetchPlan<TE
         if (K_CHUNKS % TEAM != 0 && (int)threadIdx.x + i * TEAM >= K_CHUNKS) break;
         const int key = min(max(kb + plan.k_key[i], t_lo), t_hi);
         const int key0 = min(max(kb + plan.v_key[i], v_lo), v_hi);
-        const size_t page_at = (size_t)(unsigned)pages_get(pages, key >> ps_log2) * page_stride;
+        const size_t page_at = (size_t)(unsigned)page[i] * page_stride;
         t.k[i] = *reinterpret_cast<const u32x4*>(kp + page_at + (unsigned)(plan.k_off[i] + (key & ps_mask) * HD));
         t.v[i] = *reinterpret_cast<const u32x4*>(vp + page_at + (unsigned)(plan.v_off[i] + (key0 & ps_mask)));
     }
@@ -799,6 +815,8 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
         constexpr int STEP_KEYS = KTILES * TILE;
         constexpr int AHEAD = PF_NQ == 1 ? 4 : 2;
         constexpr bool EARLY = KSPLIT == 2 || KTILES == 1;  // all shapes but the one of 256 tokens
+        constexpr bool ONE_TILE = KSPLIT == KTILES;         // a wave takes one tile of a step (tile `part`)
+        static_assert(ONE_TILE || KSPLIT == 1, "either each set of waves takes one tile of a step, or every wave all");
         static_assert(AHEAD % 2 == 0, "the LDS stage of a step is its parity within a group of AHEAD");
         FetchPlan<TEAM> plan;
         plan.make(ps_log2, hk);
@@ -814,27 +832,40 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
             PageWindow pages;
             pages_load(pages, table, table_width, first_page, lane);
             TileRegs<TEAM> regs[AHEAD][KTILES];
-// One step: issue the loads of the tiles AHEAD steps ahead into FREE (whose tiles are in LDS by now), compute this
-// wave's tile of the step at KB from LDS stage STAGE, write the tiles that wait in NEXT (loaded AHEAD - 1 steps
-// ago) into the other stage.  With AHEAD = 4 a load has three steps' time to arrive before anybody waits for it:
+            int found[KTILES][TileRegs<TEAM>::PER_THREAD];  // pages of the tiles whose loads are issued next
+// One step: issue the loads of the tiles AHEAD steps ahead into FREE (whose tiles are in LDS by now; their pages
+// were looked up a step ago) and look up the pages for the loads of the step after, compute this wave's tile of the
+// step at KB from LDS stage STAGE, write the tiles that wait in NEXT (loaded AHEAD - 1 steps ago) into the other
+// stage.  With AHEAD = 4 a load has three steps' time to arrive before anybody waits for it:
 // with the one or two workgroups a compute unit holds when a prompt is short, nothing else would hide its latency
 // (the shapes of 32 tokens a wave have no registers to spare for it and hide it by their number).  (Macros, not
 // lambdas: register sets that a closure captures by reference end up in scratch memory.)
+#define PF_LOOKUP(KB)                                                                                           \
+    _Pragma("unroll") for (int p = 0; p < KTILES; ++p)                                                          \
+        tile_lookup<TEAM>(found[p], plan, pages, ps_log2, min((KB) + p * TILE, w_last), blk_lo, blk_hi)
 #define PF_FETCH(SET, KB)                                                                                       \
     _Pragma("unroll") for (int p = 0; p < KTILES; ++p)                                                          \
-        tile_fetch(SET[p], plan, kp, vp, pages, ps_log2, page_stride, min((KB) + p * TILE, w_last), blk_lo, blk_hi)
+        tile_fetch(SET[p], plan, kp, vp, found[p], ps_log2, page_stride, min((KB) + p * TILE, w_last), blk_lo, blk_hi)
 #define PF_STORE(SET, KB, STAGE)                                                                                \
     _Pragma("unroll") for (int p = 0; p < KTILES; ++p)                                                          \
         if ((KB) + p * TILE <= w_last) tile_store(SET[p], PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), ps_log2)
+#define PF_LIVE(MY_KB) (wave_live && (MY_KB) <= w_last && (MY_KB) <= wave_hi && (MY_KB) + TILE - 1 >= wave_lo)
 #define PF_STEP(FREE, NEXT, KB, STAGE)                                                                          \
     do {                                                                                                        \
         PF_FETCH(FREE, (KB) + AHEAD * STEP_KEYS);                                                               \
-        _Pragma("unroll") for (int p = 0; p < KTILES; ++p) {                                                    \
-            if (p % KSPLIT != part) continue; /* each set of waves its tiles of the step */                     \
-            const int my_kb = (KB) + p * TILE;                                                                  \
-            if (wave_live && my_kb <= w_last && my_kb <= wave_hi && my_kb + TILE - 1 >= wave_lo)                \
-                compute_from_lds<PF_NQ, EARLY>(PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), qf, my_kb, lo, hi, scale, \
-                                               sm, acc);                                                        \
+        PF_LOOKUP((KB) + (AHEAD + 1) * STEP_KEYS);                                                              \
+        if (ONE_TILE) { /* the wave's tile is chosen by an address, so that both sets of waves run the same code */ \
+            const int mine = KSPLIT == 2 ? part : 0, my_kb = (KB) + mine * TILE;                                \
+            if (PF_LIVE(my_kb))                                                                                 \
+                compute_from_lds<PF_NQ, EARLY>(PF_K_LDS(STAGE, mine), PF_V_LDS(STAGE, mine), qf, my_kb, lo, hi, \
+                                               scale, sm, acc);                                                 \
+        } else {                                                                                                \
+            _Pragma("unroll") for (int p = 0; p < KTILES; ++p) {                                                \
+                const int my_kb = (KB) + p * TILE;                                                              \
+                if (PF_LIVE(my_kb))                                                                             \
+                    compute_from_lds<PF_NQ, EARLY>(PF_K_LDS(STAGE, p), PF_V_LDS(STAGE, p), qf, my_kb, lo, hi,   \
+                                                   scale, sm, acc);                                             \
+            }                                                                                                   \
         }                                                                                                       \
         PF_STORE(NEXT, (KB) + STEP_KEYS, (STAGE) ^ 1);                                                          \
         __syncthreads();                                                                                        \
@@ -842,7 +873,11 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
             // steps past the last tile (to fill a group of AHEAD) load the last tile again, compute and store
             // nothing and keep the barriers in step
 #pragma unroll
-            for (int j = 0; j < AHEAD; ++j) PF_FETCH(regs[j], w_first + j * STEP_KEYS);
+            for (int j = 0; j < AHEAD; ++j) {
+                PF_LOOKUP(w_first + j * STEP_KEYS);
+                PF_FETCH(regs[j], w_first + j * STEP_KEYS);
+            }
+            PF_LOOKUP(w_first + AHEAD * STEP_KEYS);
             PF_STORE(regs[0], w_first, 0);
             __syncthreads();
             for (int kb = w_first; kb <= w_last; kb += AHEAD * STEP_KEYS) {
@@ -851,8 +886,10 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
                     PF_STEP(regs[j], regs[(j + 1) % AHEAD], kb + j * STEP_KEYS, j & 1);
             }
 #undef PF_STEP
+#undef PF_LIVE
 #undef PF_STORE
 #undef PF_FETCH
+#undef PF_LOOKUP
         }
 #undef PF_K_LDS
 #undef PF_V_LDS
