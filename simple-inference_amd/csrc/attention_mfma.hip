@@ -1091,32 +1091,58 @@ static int launch_prefill(int tiles, const void* q, int q_row_stride, const void
     return SIA_LAUNCH_CHECK();
 }
 
+// Which of the four workgroup shapes a launch takes.  n_tiles, n_tiles_split, n_tiles_long: its row tiles at 128, 64
+// and 256 tokens a workgroup; q_bound, kv_bound: the most tokens and the most keys of one of its sequences (0: not
+// known, taken as a prompt from its start).
+enum PrefillShape { PF_SPLIT, PF_PAIRED, PF_WIDE, PF_LONG };
+static PrefillShape prefill_shape(int n_tiles, int n_tiles_split, int n_tiles_long, int n_heads, int q_bound,
+                                  int kv_bound) {
+    // Measured at 24 heads of 128 on 256 compute units.  For a prompt from its start, whose row tiles see from few
+    // keys to all, the fastest shape follows the number of workgroups per compute unit: the split shape while all
+    // its workgroups are on the chip at once (up to 6/8 of a wide workgroup per compute unit: prompts up to about
+    // 1,000 tokens), the paired shape of 128 tokens (two tiles of keys a step, one for each set of waves) up to 15/8
+    // (about 2,500 tokens), the wide shape (one tile a step) beyond, and from 36/8 on (about 6,000 tokens) 8 waves
+    // of 32 tokens (256 tokens a workgroup, two tiles a step: a tile staged in LDS then serves twice as many tokens).
+    const long long wide_groups = (long long)n_tiles * n_heads, cus = compute_units();
+    const bool split_fits = n_tiles_split > 0 && wide_groups * 8 <= cus * 6;
+    // A portion over a past is another matter: every row tile sees about as many keys, so the launch lasts as many
+    // rounds as its workgroups need on the compute units, each as long as the shape's time for that many keys.
+    if (split_fits && q_bound > 0 && 2LL * kv_bound >= 3LL * q_bound && (long long)n_tiles_split * n_heads > cus)
+        return PF_PAIRED;  // one round of 128 tokens instead of two of 64 (768 to 1,024 tokens: 10 to 30 % less)
+    if (!split_fits && q_bound > 0 && kv_bound >= 4LL * q_bound) {
+        // time of a round for a given number of keys, relative: a compute unit holds one paired workgroup (128
+        // tokens), two wide ones (256) or one long one (256)
+        const long long paired = (wide_groups + cus - 1) / cus * 124;
+        const long long wide = (wide_groups + 2 * cus - 1) / (2 * cus) * 236;
+        const long long lng = n_tiles_long > 0 ? ((long long)n_tiles_long * n_heads + cus - 1) / cus * 222 : paired + wide;
+        return lng <= wide && lng <= paired ? PF_LONG : wide <= paired ? PF_WIDE : PF_PAIRED;
+    }
+    if (split_fits) return PF_SPLIT;
+    if (wide_groups * 8 <= cus * 15) return PF_PAIRED;
+    if (n_tiles_long > 0 && wide_groups * 8 >= cus * 36) return PF_LONG;
+    return PF_WIDE;
+}
+
 SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                                 const int* block_table, int table_width, const int* cu_q, const int* kv_len,
                                 void* out, int seq_begin, int seq_end, int n_tiles, int n_tiles_split, int n_tiles_long,
-                                int n_heads, int n_kv, int page_size, float scale, int window, hipStream_t stream) {
+                                int q_bound, int kv_bound, int n_heads, int n_kv, int page_size, float scale, int window,
+                                hipStream_t stream) {
     if (seq_end <= seq_begin || n_tiles <= 0) return 0;
     const int ps_log2 = log2_exact(page_size);
     if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads > 65535 || q_row_stride % 8 || table_width <= 0)
         return SIA_BAD_ARGUMENT;
 #define ARGS q, q_row_stride, k_pages, v_pages, block_table, table_width, cu_q, kv_len, out, seq_begin, seq_end, \
              n_heads, n_kv, ps_log2, scale, window, stream
-    if constexpr (HD > 128) {
-        return launch_prefill<1, PF_ROWS / 16, 1>(n_tiles, ARGS);
+    if constexpr (HD > 128 || !PF_USE_LDS) {
+        return HD > 128 ? launch_prefill<1, PF_ROWS / 16, 1>(n_tiles, ARGS) : launch_prefill<2, PF_ROWS / 32, 1>(n_tiles, ARGS);
     } else {
-        // Which shape is the fastest follows the number of workgroups per compute unit (measured at 24 heads of 128
-        // on 256 compute units): the split shape while all its workgroups are on the chip at once (up to 6/8 of a
-        // wide workgroup per compute unit: prompts or portions up to about 1,000 tokens), the paired shape of 128
-        // tokens (two tiles of keys a step, one for each set of waves) up to 15/8 (about 2,500 tokens), the wide
-        // shape (one tile a step) beyond, and from 36/8 on (about 6,000 tokens) 8 waves of 32 tokens (256 tokens a
-        // workgroup, two tiles a step: a tile staged in LDS then serves twice as many tokens).
-        const long long wide_groups = (long long)n_tiles * n_heads, cus = compute_units();
-        if (PF_USE_LDS && n_tiles_split > 0 && wide_groups * 8 <= cus * 6)
-            return launch_prefill<1, 2 * PF_ROWS_SPLIT / 16, 2>(n_tiles_split, ARGS);
-        if (PF_USE_LDS && wide_groups * 8 <= cus * 15) return launch_prefill<2, 2 * PF_ROWS / 32, 2, 2>(n_tiles, ARGS);
-        if (PF_USE_LDS && n_tiles_long > 0 && wide_groups * 8 >= cus * 36)
-            return launch_prefill<2, PF_ROWS_LONG / 32, 1, 2>(n_tiles_long, ARGS);
-        return launch_prefill<2, PF_ROWS / 32, 1>(n_tiles, ARGS);
+        switch (prefill_shape(n_tiles, n_tiles_split, n_tiles_long, n_heads, q_bound, kv_bound)) {
+            case PF_SPLIT: return launch_prefill<1, 2 * PF_ROWS_SPLIT / 16, 2>(n_tiles_split, ARGS);
+            case PF_PAIRED: return launch_prefill<2, 2 * PF_ROWS / 32, 2, 2>(n_tiles, ARGS);
+            case PF_LONG: return launch_prefill<2, PF_ROWS_LONG / 32, 1, 2>(n_tiles_long, ARGS);
+            default: return launch_prefill<2, PF_ROWS / 32, 1>(n_tiles, ARGS);
+        }
     }
 #undef ARGS
 }

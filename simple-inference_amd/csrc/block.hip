@@ -22,8 +22,9 @@ typedef int (*DecodeFn)(const void* q, int q_row_stride, const void* k_pages, co
                         int window, int max_splits, hipStream_t stream);
 typedef int (*PrefillFn)(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                          const int* block_table, int table_width, const int* cu_q, const int* kv_len, void* out,
-                         int seq_begin, int seq_end, int n_tiles, int n_tiles_split, int n_tiles_long, int n_heads,
-                         int n_kv, int page_size, float scale, int window, hipStream_t stream);
+                         int seq_begin, int seq_end, int n_tiles, int n_tiles_split, int n_tiles_long, int q_bound,
+                         int kv_bound, int n_heads, int n_kv, int page_size, float scale, int window,
+                         hipStream_t stream);
 
 // What a block owns: its weights (bfloat16 matrices [out, in], float gains) and its constants.
 struct SiaBlockOwn {
@@ -59,7 +60,7 @@ struct SiaBlockStep {
     const int* kv_len;
     float* ws_acc;
     float* ws_ml;
-    int n_tokens, n_seqs, n_single, max_splits, n_tiles, n_tiles_split, n_tiles_long;
+    int n_tokens, n_seqs, n_single, max_splits, n_tiles, n_tiles_split, n_tiles_long, q_bound, kv_bound;
 };
 
 #define SIA_STEP(call)             \
@@ -90,7 +91,7 @@ SIA_EXPORT int sia_prenorm_block(const SiaBlockOwn* B, const SiaBlockStep* S, co
     if (S->n_single < S->n_seqs)
         SIA_STEP(S->attend_runs(S->qkv, qkv_width, k_pages, v_pages, block_table, table_width, S->cu_q, S->kv_len,
                                 S->attended, S->n_single, S->n_seqs, S->n_tiles, S->n_tiles_split, S->n_tiles_long,
-                                B->n_heads, B->n_kv, page_size, B->scale, B->window, stream));
+                                S->q_bound, S->kv_bound, B->n_heads, B->n_kv, page_size, B->scale, B->window, stream));
     SIA_STEP(S->product(S->attended, B->w_o, S->mixed, M, H, Q, 0, stream));
     SIA_STEP(sia_add_rmsnorm(S->residual, S->mixed, B->feed_forward_norm_gain, S->normed, nullptr, M, H,
                              B->feed_forward_norm_eps, SIA_BF16, stream));

@@ -178,6 +178,7 @@ class StepRunner:
             state_slots=part(5), logit_rows=part(6)[:n_rows] if n_rows else None, n_logit_rows=n_rows,
             max_q_len=max(q_lens), max_kv_len=int(kvl.max()), kernels=self.kernels,
             n_decode_seqs=n_decode, q_lens=q_lens,
+            max_run_kv_len=int(kvl[n_decode:].max()) if n_decode < n_seqs else 0,
         )
         ctx.block_tables = [part(7 + g).view(n_seqs, width) for g in range(n_groups)]
         ctx.extra = {key: part(9 + n_groups + i) for i, key in enumerate(extra_keys)}

@@ -59,7 +59,8 @@ _ATTN_SIGNATURES = {
     "sia_attn_decode": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                         _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_attn_prefill": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
-                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                         _c_ptr],
     "sia_attn_decode_max_splits": [_c_int, _c_int],
     "sia_attn_decode_workspace": [_c_int, _c_int, _c_int, _c_int, _c_int],
     "sia_attn_decode_mode": [_c_int, _c_int, _c_int, _c_int],
@@ -125,7 +126,7 @@ class _BlockStep(ctypes.Structure):
                                                "attended", "mixed", "gate_up", "activated", "fed", "positions",
                                                "seq_of_token", "cu_q", "kv_len", "ws_acc", "ws_ml")]
                 + [(n, ctypes.c_int) for n in ("n_tokens", "n_seqs", "n_single", "max_splits", "n_tiles", "n_tiles_split",
-                                               "n_tiles_long")])
+                                               "n_tiles_long", "q_bound", "kv_bound")])
 
 
 def _bind(lib, signatures):
@@ -562,11 +563,14 @@ class HipKernels:
                 torch.empty((floats,), dtype=torch.float32, device=device) if floats else None
                 for floats in (lib.sia_attn_decode_workspace(n_dec, n_heads, n_kv_heads, max_splits, which)
                                for which in (0, 1)))
-        tiles = (0, 0, 0)
+        tiles = (0, 0, 0, 0, 0)
         if n_dec < ctx.n_seqs:
+            # row tiles at each of the kernel's workgroup sizes, and what bounds a sequence's tokens and keys in this
+            # step: a portion over a long past takes another workgroup shape than a prompt from its start
             tiles = tuple(sum(-(-q // rows) for q in ctx.q_lens[n_dec:]) if rows else 0
                           for rows in (lib.sia_attn_prefill_rows(), lib.sia_attn_prefill_rows_split(),
                                        lib.sia_attn_prefill_rows_long()))
+            tiles += (int(max(ctx.q_lens[n_dec:])), int(getattr(ctx, "max_run_kv_len", 0) or ctx.max_kv_len))
         plan = (n_dec, max_splits, ws_acc, ws_ml, tiles)
         if plans is None:
             try:
@@ -580,8 +584,8 @@ class HipKernels:
         lib = self._attn_lib(head_dim)
         width = qkv.shape[1]
         table = cache.block_table
-        n_dec, max_splits, ws_acc, ws_ml, (n_tiles, n_tiles_split, n_tiles_long) = self._attention_plan(
-            lib, qkv.device, n_heads, n_kv_heads, head_dim, window, ctx)
+        n_dec, max_splits, ws_acc, ws_ml, (n_tiles, n_tiles_split, n_tiles_long, q_bound, kv_bound) = \
+            self._attention_plan(lib, qkv.device, n_heads, n_kv_heads, head_dim, window, ctx)
         if n_dec:
             self._check(lib.sia_attn_decode(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
@@ -591,8 +595,9 @@ class HipKernels:
         if n_dec < ctx.n_seqs:
             self._check(lib.sia_attn_prefill(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
-                _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_tiles_split, n_tiles_long, n_heads,
-                n_kv_heads, cache.page_size, float(scale), window, self._stream()), "attn_prefill")
+                _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_tiles_split, n_tiles_long,
+                q_bound, kv_bound, n_heads, n_kv_heads, cache.page_size, float(scale), window, self._stream()),
+                "attn_prefill")
 
     # -- a whole block in one call -------------------------------------------------
     def _library_can(self, M, N, K) -> bool:

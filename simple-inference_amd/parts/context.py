@@ -47,6 +47,7 @@ class StepContext:
     n_decode_seqs: int = 0  # sequences 0 .. n_decode_seqs-1 bring exactly one token (they are sorted first)
     q_lens: list = field(default_factory=list)  # host copy: tokens each sequence brings
     kv_bound: int = 0  # replayed graphs: an upper bound of kv_len that fixes grids (0: use max_kv_len)
+    max_run_kv_len: int = 0  # the longest kv_len among the sequences that bring more than one token (0: not known)
     extra: dict = field(default_factory=dict)  # name -> int32 [n_tokens]: what the step's entries brought beside tokens
 
 
