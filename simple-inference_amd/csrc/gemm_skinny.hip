@@ -89,7 +89,10 @@ struct Epilogue {
 // the gate half and row u of the up half of W), or a pair of columns that the rotation mixes (EPI_ROPE: unit u is
 // column u % (head_dim / 2) of head u / (head_dim / 2) together with the column head_dim / 2 further).  A workgroup
 // owns UNIT_BLOCKS blocks of bh consecutive units from blockIdx.x * UNIT_BLOCKS * bh on.
-template <typename TOut, int RB, int WAVES, int EPI, bool SCALED>
+// TILED: W is not [N][K] but a copy laid out for this cut, so that every load instruction of a wave reads one
+// run of memory: [block of bh rows][step of 64 k][half of a lane's 16 k][row][lane group][8 k] (see
+// sia_gemm_skinny_tiled_weights).  The same elements meet in the same products, so no bit changes.
+template <typename TOut, int RB, int WAVES, int EPI, bool SCALED, bool TILED = false>
 __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                      const bf16_t* __restrict__ W,
                                                                      TOut* __restrict__ Y, int M, int N, int K,
@@ -122,7 +125,10 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
             row = unit_at(rb % UNIT_BLOCKS, r) + (rb / UNIT_BLOCKS) * N;
         }
         w_row[rb] = W + (size_t)row * K + g * 16;
+        if (TILED)  // the block's tiles: (step, half) apart by bh * 32 elements, this lane's piece inside a tile
+            w_row[rb] = W + (size_t)(blockIdx.x * RB + rb) * (K / SK_STEP) * 2 * bh * 32 + (min(r, bh - 1) * 4 + g) * 8;
     }
+    static_assert(!TILED || EPI == EPI_STORE || EPI == EPI_RESIDUAL, "tiled weights: a row block is a block of columns");
 
     // requested before the weights, used after them.  The sums of squares of a row are added up the way the
     // products are: 64 runners (16 shares of 4 lane groups), runner l taking partials l, l + 64, ...
@@ -173,8 +179,14 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
                 if (k + u * SK_STEP < K) {
 #pragma unroll
                     for (int rb = 0; rb < RB; ++rb) {
-                        a[u][rb][0] = ld8(w_row[rb] + k + u * SK_STEP);
-                        a[u][rb][1] = ld8(w_row[rb] + k + u * SK_STEP + 8);
+                        if (TILED) {
+                            const size_t tile = (size_t)((k / SK_STEP + u) * 2) * bh * 32;
+                            a[u][rb][0] = ld8(w_row[rb] + tile);
+                            a[u][rb][1] = ld8(w_row[rb] + tile + bh * 32);
+                        } else {
+                            a[u][rb][0] = ld8(w_row[rb] + k + u * SK_STEP);
+                            a[u][rb][1] = ld8(w_row[rb] + k + u * SK_STEP + 8);
+                        }
                     }
                     b[u][0] = ld8(x_row + k + u * SK_STEP);
                     b[u][1] = ld8(x_row + k + u * SK_STEP + 8);
@@ -392,6 +404,29 @@ SIA_EXPORT int sia_gemm_skinny_residual(const void* X, const void* W, int M, int
     Epilogue ep{};
     ep.res = ResidualOut{residual, gain, (bf16_t*)scaled, partials};
     launch_skinny<bf16_t, EPI_RESIDUAL>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, ep, stream);
+    return SIA_LAUNCH_CHECK();
+}
+
+// The tiled copy of W[N][K] that sia_gemm_skinny_residual_tiled reads: sia_gemm_skinny_tile_height(N) rows a block
+// (0: this N is cut into workgroups of several blocks, which have no tiled form), blocks = ceil(N / height), the
+// last block's missing rows repeating row N - 1; elements [block][K / 64][2][height][4][8], where element
+// (b, s, h, r, g, e) is W[b * height + r][64 s + 16 g + 8 h + e].
+SIA_EXPORT int sia_gemm_skinny_tile_height(int N) {
+    if (N <= 0) return 0;
+    const Cut cut = cheapest(N, 1, {4, 2, 1});
+    return cut.unit_blocks == 1 ? cut.bh : 0;
+}
+
+SIA_EXPORT int sia_gemm_skinny_residual_tiled(const void* X, const void* W_tiled, int M, int N, int K, float* residual,
+                                              const float* gain, void* scaled, float* partials, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 64 || K <= 0 || !residual || !gain || !scaled || !partials) return SIA_BAD_ARGUMENT;
+    const Cut cut = cheapest(N, 1, {4, 2, 1});
+    if (cut.unit_blocks != 1) return SIA_BAD_ARGUMENT;
+    Epilogue ep{};
+    ep.res = ResidualOut{residual, gain, (bf16_t*)scaled, partials};
+    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 1, 8, EPI_RESIDUAL, false, true>), dim3(cut.grid), dim3(8 * SIA_WAVE), 0,
+                       stream, (const bf16_t*)X, (const bf16_t*)W_tiled, (bf16_t*)nullptr, M, N, K, cut.bh, ep);
     return SIA_LAUNCH_CHECK();
 }
 

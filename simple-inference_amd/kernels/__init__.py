@@ -49,6 +49,8 @@ _SIGNATURES = {
     "sia_gemm_skinny_rope": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
                              _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_ptr],
     "sia_gemm_skinny_residual": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "sia_gemm_skinny_residual_tiled": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "sia_gemm_skinny_tile_height": [_c_int],
     "sia_place_tokens": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "sia_scale_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr],
     "sia_stream_read": [_c_ptr, _c_ll, _c_ptr, _c_ptr],
@@ -153,6 +155,7 @@ class HipKernels:
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self._device_index = torch.device(device).index or 0
         self.use_mfma_attention = True   # tests switch it off to reach the plain kernel in bfloat16
+        self.tiled_weights = True        # tests switch it off to compare with the product that reads W as it is
         self.use_skinny_gemm = True      # few-row bfloat16 products by this package's kernel, not the library
         self.fuse_norms = True           # few rows: residual add in the product before a norm, row scale in the one after
         self.fuse_rope = True            # few rows: rotation and cache write in the q/k/v product
@@ -380,10 +383,43 @@ class HipKernels:
                               f"residual {tuple(residual.shape)}, gain {tuple(gain.shape)}")
         rows = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
         partials = torch.empty((self.core.sia_gemm_skinny_residual_blocks(N), 16), dtype=torch.float32, device=x.device)
-        self._check(self.core.sia_gemm_skinny_residual(_ptr(x), _ptr(w), M, N, K, _ptr(residual), _ptr(gain),
-                                                       _ptr(rows), _ptr(partials), self._stream()),
-                    "gemm_skinny_residual")
+        tiled = self._tiled_copy(w)
+        if tiled is not None:
+            self._check(self.core.sia_gemm_skinny_residual_tiled(_ptr(x), _ptr(tiled), M, N, K, _ptr(residual),
+                                                                 _ptr(gain), _ptr(rows), _ptr(partials), self._stream()),
+                        "gemm_skinny_residual_tiled")
+        else:
+            self._check(self.core.sia_gemm_skinny_residual(_ptr(x), _ptr(w), M, N, K, _ptr(residual), _ptr(gain),
+                                                           _ptr(rows), _ptr(partials), self._stream()),
+                        "gemm_skinny_residual")
         return ScaledRows(rows, partials, float(eps))
+
+    # A weight whose product goes into the residual in steps of few rows may have a second copy, laid out in the
+    # order in which that kernel's workgroups read it (every load instruction one run of memory: the o and down
+    # products of a decode step take 10 to 15 % less).  The copy hangs on the weight tensor itself, so it lives as long
+    # as the weight does, and remembers the version of the tensor it was made from: a weight changed in place since
+    # is read as it is.  Steps of more rows, which go to the library, read the weight as it is anyway.
+    def prepare_pending_weight(self, w) -> bool:
+        """Makes the tiled copy of a weight that ``pending_linear`` will be given; True if one was made."""
+        if (not self.tiled_weights or not isinstance(w, torch.Tensor) or w.dim() != 2 or w.dtype != torch.bfloat16
+                or not w.is_cuda or not w.is_contiguous() or w.shape[1] % 64 or torch.cuda.is_current_stream_capturing()):
+            return False
+        N, K = w.shape
+        height = self.core.sia_gemm_skinny_tile_height(N)
+        if height <= 0:
+            return False
+        blocks = -(-N // height)
+        rows = torch.arange(blocks * height, device=w.device).clamp_(max=N - 1)   # the last block repeats the last row
+        # element (block, step, half, row, lane group, e) = W[block * height + row][64 step + 16 group + 8 half + e]
+        tiled = w[rows].view(blocks, height, K // 64, 4, 2, 8).permute(0, 2, 4, 1, 3, 5).contiguous()
+        w._sia_tiled = (tiled, w._version)
+        return True
+
+    def _tiled_copy(self, w):
+        kept = getattr(w, "_sia_tiled", None) if self.tiled_weights else None
+        if kept is None or kept[1] != w._version:
+            return None
+        return kept[0]
 
     @staticmethod
     def _scaled(x):

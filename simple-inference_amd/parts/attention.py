@@ -82,6 +82,9 @@ class Attention:
         else:
             self.w_qkv = tensors["q"].contiguous()
         self.w_o = tensors["o"].contiguous()
+        prepare = getattr(self.env.kernels, "prepare_pending_weight", None)
+        if prepare is not None:   # the kernels may keep a copy of their own of a weight whose product is left pending
+            prepare(self.w_o)
 
     def plain_form(self):
         """What this mixer is, as plain data, for kernels that can run a whole block in one call; None for the forms

@@ -37,6 +37,9 @@ class SwiGLU:
     def bind(self, tensors):
         self.w_gate_up = torch.cat([tensors["gate"], tensors["up"]], dim=0).contiguous()
         self.w_down = tensors["down"].contiguous()
+        prepare = getattr(self.env.kernels, "prepare_pending_weight", None)
+        if prepare is not None:   # the kernels may keep a copy of their own of a weight whose product is left pending
+            prepare(self.w_down)
 
     def plain_form(self):
         """What this feed-forward is, as plain data, for kernels that can run a whole block in one call (None for

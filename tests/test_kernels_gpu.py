@@ -513,6 +513,41 @@ def test_few_row_products_do_not_depend_on_the_number_of_rows(hip):
             assert torch.equal(got, want[:m]), m
 
 
+@pytest.mark.parametrize("N, K", [(3072, 3072), (3070, 8192), (2048, 2048), (4099, 192)])
+def test_a_tiled_copy_of_a_weight_changes_no_bit_of_the_product_into_the_residual(hip, N, K):
+    """The product into the residual reads, where the kernels made one, a copy of the weight laid out in the order
+    of its loads.  The same elements meet in the same sums: residual, scaled rows and sums of squares are the same
+    bit for bit as from the weight as it is, for every number of rows, also where the last block of rows is short
+    (3,070 and 4,099 rows).  A weight changed in place after the copy was made is read as it is."""
+    dtype = torch.bfloat16
+    x = rnd(16, K, dtype=dtype, seed=1)
+    w = rnd(N, K, dtype=dtype, seed=2, scale=K ** -0.5)
+    res = rnd(16, N, seed=3, scale=2.0)
+    gain = (rnd(N, seed=4, scale=0.3) + 1.0).contiguous()
+
+    def through(m):
+        r = res[:m].clone()
+        scaled = hip.linear_into_residual(hip.pending_linear(x[:m].contiguous(), w), r, gain, 1e-5)
+        return r, scaled.rows, scaled.partials[:, :m].clone()
+
+    plain = {m: through(m) for m in (1, 7, 16)}
+    made = hip.prepare_pending_weight(w)
+    assert made == (hip.core.sia_gemm_skinny_tile_height(N) > 0)
+    for m, want in plain.items():
+        for got, expected in zip(through(m), want):
+            assert torch.equal(got, expected), (N, K, m)
+    if made:
+        assert hip._tiled_copy(w) is not None
+        w.mul_(2.0)                                    # the copy no longer says what the weight holds
+        assert hip._tiled_copy(w) is None
+        r, rows, _ = through(5)
+        want = res[:5] + (x[:5].float() @ w.float().T).to(dtype).float()
+        torch.testing.assert_close(r, want, atol=2e-2, rtol=2e-2)
+        assert hip.prepare_pending_weight(w) and hip._tiled_copy(w) is not None
+        for got, expected in zip(through(5), (r, rows)):
+            assert torch.equal(got, expected)
+
+
 @pytest.mark.parametrize("q_len, kv_len, window", [(130, 130, None), (900, 1000, None), (1900, 1900, None),
                                                   (1900, 2100, 300)])
 def test_matrix_core_prefill_in_each_workgroup_shape(hip, q_len, kv_len, window):

@@ -225,8 +225,8 @@ def test_few_token_steps_take_the_products_with_fused_epilogues(folders):
     tiny = TINIES["d"]
     runner, cache, mcfg = make_runner(folders["d"], "hip-bf16", tiny.page_size, num_pages=64)
     core = runner.kernels.core
-    counted = ("sia_gemm_skinny_rope", "sia_gemm_skinny_residual", "sia_gemm_skinny_swiglu", "sia_rope_kv_write",
-               "sia_add_rmsnorm", "sia_prenorm_block")
+    counted = ("sia_gemm_skinny_rope", "sia_gemm_skinny_residual", "sia_gemm_skinny_residual_tiled",
+               "sia_gemm_skinny_swiglu", "sia_rope_kv_write", "sia_add_rmsnorm", "sia_prenorm_block")
     calls = {name: 0 for name in counted}
     real = {name: getattr(core, name) for name in counted}
 
@@ -244,6 +244,7 @@ def test_few_token_steps_take_the_products_with_fused_epilogues(folders):
         cache.admit("r")
         runner.run([StepEntry("r", tokens[:20], [19])])       # many tokens: the library's products, separate kernels,
         assert calls["sia_gemm_skinny_rope"] == calls["sia_gemm_skinny_residual"] == 0    # launched by one call a layer
+        assert calls["sia_gemm_skinny_residual_tiled"] == 0
         assert calls["sia_prenorm_block"] == layers and calls["sia_rope_kv_write"] == 0 and calls["sia_add_rmsnorm"] == 1
         for name in counted:
             calls[name] = 0
@@ -251,12 +252,14 @@ def test_few_token_steps_take_the_products_with_fused_epilogues(folders):
         runner.run([StepEntry("r", tokens[20:37], [16])])
         runner.kernels.whole_blocks = True
         assert calls["sia_gemm_skinny_rope"] == calls["sia_gemm_skinny_residual"] == calls["sia_prenorm_block"] == 0
+        assert calls["sia_gemm_skinny_residual_tiled"] == 0
         assert calls["sia_rope_kv_write"] == layers and calls["sia_add_rmsnorm"] == 2 * layers + 1
         for name in counted:
             calls[name] = 0
         runner.run([StepEntry("r", tokens[37:], [2])])        # three tokens
         assert calls["sia_gemm_skinny_rope"] == layers and calls["sia_gemm_skinny_swiglu"] == layers
-        assert calls["sia_gemm_skinny_residual"] == 2 * layers - 1   # the last product waits for the rows that are wanted
+        # (from the weight as it is or from the kernels' own copy of it; the last product waits for the rows that are wanted)
+        assert calls["sia_gemm_skinny_residual"] + calls["sia_gemm_skinny_residual_tiled"] == 2 * layers - 1
         assert calls["sia_rope_kv_write"] == 0 and calls["sia_add_rmsnorm"] == 2   # the first norm and the last
     finally:
         for name in counted:
